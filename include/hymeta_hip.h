@@ -26,7 +26,8 @@
  *  - hymeta_abi_version() returns the HYMETA_ABI_VERSION the library was built
  *    with; a binding compares it with the header it was written against before
  *    the first call (version 2: every argument struct starts with struct_size;
- *    version 3: hymeta_gla_decode_args ends with qkv_x_scale / qkv_w_scale).
+ *    version 3: hymeta_gla_decode_args ends with qkv_x_scale / qkv_w_scale;
+ *    version 4: the recurrent / biased-attention building blocks at the end of this file).
  *  - Every argument struct starts with `uint32_t struct_size`, which the caller
  *    sets to sizeof(the struct) of ITS declaration.  An entry point returns
  *    HYMETA_ERR_INVALID_ARG, before it reads any other field, when the value
@@ -44,7 +45,7 @@
 extern "C" {
 #endif
 
-#define HYMETA_ABI_VERSION 3
+#define HYMETA_ABI_VERSION 4
 
 typedef void* hymeta_stream_t;
 
@@ -1053,6 +1054,183 @@ int hymeta_p2p_all_reduce_partials(hymeta_p2p_comm* comm, const hymeta_gemm_part
                                    hymeta_stream_t stream);
 int hymeta_p2p_timeouts(hymeta_p2p_comm* comm, uint32_t* count);
 int hymeta_p2p_destroy(hymeta_p2p_comm* comm);
+
+/* ============================================================================================
+ * Building blocks of recurrent / biased-attention decoder designs (first user: the Sonuzen model
+ * class).  Nothing here has a counterpart in the reference.  Every entry point takes `act_dtype`,
+ * HYMETA_BF16 or HYMETA_F32: the type of the activations, the paged K/V rows and the convolution
+ * state.  Norm statistics, softmax scores and weights, recurrent states and the residual stream are
+ * fp32 in both.  Small parameter vectors (norm weights, convolution taps, biases, per-head constants)
+ * are fp32.
+ *
+ * A step's tokens are laid out sequence after sequence: sequence s owns rows
+ * query_start_loc[s] .. query_start_loc[s + 1] - 1; context_lens[s] tokens of it were processed by
+ * earlier steps (0: the sequence starts here and every carried state reads as zero, so a slot that
+ * another sequence used before needs no clearing); slot_idx[s] is its state slot (-1: none, state
+ * neither read nor written).
+ * ========================================================================================== */
+
+/* out[t] = table[token_ids[t]] (+ add), fp32 rows: the start of an fp32 residual stream. */
+typedef struct hymeta_embed_rows_args {
+  uint32_t struct_size;
+  const int64_t* token_ids;    /* [num_tokens] */
+  const void* table;           /* act_dtype [vocab, width] contiguous */
+  const float* add;            /* [width] or NULL */
+  float* out;                  /* [num_tokens, width] contiguous */
+  int32_t num_tokens, width, vocab, act_dtype;
+} hymeta_embed_rows_args;
+int hymeta_embed_rows(const hymeta_embed_rows_args* args, hymeta_stream_t stream);
+
+/* RMS norm of fp32 rows followed by an optional short causal convolution over time, per channel:
+ *   n[t]   = x[t] / sqrt(mean(x[t]^2) + eps) * (weight_offset + weight)      (rounded to act_dtype)
+ *   out[t] = n[t] + sum_{j < taps} conv_weight[:, j] * n[t - (taps - 1) + j]   (conv_weight NULL: out = n)
+ * with n before a sequence's first token = 0.  conv_state [slots, taps - 1, width] holds the last
+ * taps - 1 rows n of every sequence between steps; it is read for the first rows of a portion and
+ * rewritten at its end, in the same launch.  taps <= HYMETA_CONV_MAX_TAPS. */
+#define HYMETA_CONV_MAX_TAPS 8
+typedef struct hymeta_norm_conv_args {
+  uint32_t struct_size;
+  const float* x;              /* [num_tokens, width], row stride x_stride_t */
+  const float* weight;         /* [width] */
+  const float* conv_weight;    /* [width, taps] or NULL */
+  void* conv_state;            /* act_dtype [slots, taps - 1, width] or NULL */
+  void* out;                   /* act_dtype [num_tokens, width] contiguous */
+  const int32_t* query_start_loc;  /* [num_seqs + 1] */
+  const int32_t* context_lens;     /* [num_seqs] */
+  const int32_t* slot_idx;         /* [num_seqs] */
+  int32_t num_tokens, num_seqs, width, taps, act_dtype;
+  float eps, weight_offset;
+  int64_t x_stride_t;
+} hymeta_norm_conv_args;
+int hymeta_norm_conv(const hymeta_norm_conv_args* args, hymeta_stream_t stream);
+
+/* x[t] += mult * y[t] / sqrt(mean(y[t]^2) + eps) * (weight_offset + weight) (+ post_add): a sublayer's
+ * output through its output norm into the fp32 residual stream, in place. */
+typedef struct hymeta_norm_residual_args {
+  uint32_t struct_size;
+  const void* y;               /* act_dtype [num_tokens, width], row stride y_stride_t */
+  const float* weight;         /* [width] */
+  const float* post_add;       /* [width] or NULL */
+  float* x;                    /* [num_tokens, width], row stride x_stride_t */
+  int32_t num_tokens, width, act_dtype;
+  float eps, weight_offset, mult;
+  int64_t y_stride_t, x_stride_t;
+} hymeta_norm_residual_args;
+int hymeta_norm_residual(const hymeta_norm_residual_args* args, hymeta_stream_t stream);
+
+/* minGRU recurrence over a step's rows, per channel c of `width`:
+ *   z = sigmoid(zr), cand = u >= 0 ? u + 0.5 : sigmoid(u), S <- (1 - z) S + z cand, out = S * silu(g)
+ * zr, u, g: columns [0, W), [W, 2W), [2W, 3W) of `zug` (the three projections' outputs, biases
+ * included).  state fp32 [slots, width] is carried between steps. */
+typedef struct hymeta_mingru_args {
+  uint32_t struct_size;
+  const void* zug;             /* act_dtype [num_tokens, 3 * width], row stride zug_stride_t */
+  float* state;                /* [slots, width] */
+  void* out;                   /* act_dtype [num_tokens, width] contiguous */
+  const int32_t* query_start_loc;
+  const int32_t* context_lens;
+  const int32_t* slot_idx;
+  int32_t num_tokens, num_seqs, width, act_dtype, max_query_len;
+  int64_t zug_stride_t;
+} hymeta_mingru_args;
+int hymeta_mingru(const hymeta_mingru_args* args, hymeta_stream_t stream);
+
+/* Per-head RMS norm of the query and key columns of a fused q|k|v projection and the paged write of
+ * the step's keys and values:
+ *   q[t, h] <- q[t, h] / sqrt(mean(q[t, h]^2) + eps) * q_weight   (in place; k alike with k_weight)
+ *   kv_cache[slot_mapping[t]] <- (k[t], v[t])
+ * kv_cache: act_dtype [num_blocks, block_size, num_kv_heads, head_dim + v_dim], a key row followed by
+ * its value row.  q_weight / k_weight NULL: no norm.  slot_mapping[t] < 0: nothing is stored. */
+typedef struct hymeta_qk_norm_cache_args {
+  uint32_t struct_size;
+  void* qkv;                   /* act_dtype [num_tokens, H * D + G * D + G * Dv], row stride qkv_stride_t */
+  const float* q_weight;       /* [head_dim] or NULL */
+  const float* k_weight;       /* [head_dim] or NULL */
+  void* kv_cache;
+  const int64_t* slot_mapping; /* [num_tokens] */
+  int32_t num_tokens, num_heads, num_kv_heads, head_dim, v_dim, block_size, act_dtype;
+  float eps;
+  int64_t num_blocks, qkv_stride_t;
+} hymeta_qk_norm_cache_args;
+int hymeta_qk_norm_cache(const hymeta_qk_norm_cache_args* args, hymeta_stream_t stream);
+
+/* Causal attention of a step's queries over their sequences' paged keys (the step's own keys are in
+ * the cache already), with a distance bias and an optional sink:
+ *   s_ij = scale * q_i . k_j - bias(i - j),   j <= i   (and i - j <= window_left when window_left >= 0)
+ *   bias_mode HYMETA_BIAS_NONE: 0;  HYMETA_BIAS_LOG_DISTANCE: bias_a[h] * ln(1 + bias_b[h] * (i - j))
+ *   p_ij = exp(s_ij) / (sink + sum_j exp(s_ij)),  sink = 1 (a key of score 0 without a value) or 0
+ *   out_i = sum_j p_ij v_j
+ * Scores and weights are fp32 in both activation types.  Query row t of sequence s stands at position
+ * seq_lens[s] - (query_start_loc[s + 1] - t).  Sequences with one query row (decode) and portions of
+ * prompts run in the same launch sequence; `workspace` (hymeta_sink_attention_workspace_bytes) holds
+ * the partial results of long single-row sequences split over their keys. */
+enum hymeta_bias_mode { HYMETA_BIAS_NONE = 0, HYMETA_BIAS_LOG_DISTANCE = 1 };
+typedef struct hymeta_sink_attention_args {
+  uint32_t struct_size;
+  const void* q;               /* act_dtype [num_tokens, num_heads, head_dim], strides q_stride_t / head_dim */
+  const void* kv_cache;        /* as hymeta_qk_norm_cache writes it */
+  void* out;                   /* act_dtype [num_tokens, num_heads, v_dim] contiguous */
+  const int32_t* block_tables; /* [num_seqs, block_table_stride] */
+  const int32_t* query_start_loc;  /* [num_seqs + 1] */
+  const int32_t* seq_lens;         /* [num_seqs]: keys of the sequence, this step's rows included */
+  const float* bias_a;         /* [num_heads] */
+  const float* bias_b;         /* [num_heads] */
+  void* workspace;
+  size_t workspace_bytes;
+  int32_t num_tokens, num_seqs, num_heads, num_kv_heads, head_dim, v_dim, block_size, act_dtype;
+  int32_t bias_mode, sink, window_left, max_query_len, max_seq_len;
+  float scale;
+  int64_t num_blocks, q_stride_t, block_table_stride;
+} hymeta_sink_attention_args;
+size_t hymeta_sink_attention_workspace_bytes(int32_t num_tokens, int32_t num_heads, int32_t v_dim, int32_t max_seq_len);
+int hymeta_sink_attention(const hymeta_sink_attention_args* args, hymeta_stream_t stream);
+
+/* Mixture of experts whose choice is a table lookup by token id: table [vocab, top_k] names each
+ * token's experts (distinct within a row), every choice weighs 1 / top_k.  Writes what
+ * hymeta_moe_route writes (topk_ids, topk_weights, expert_offsets, sorted_pair, pair_pos), so the
+ * grouped GEMMs and the combine that follow are the routed block's.  One launch. */
+typedef struct hymeta_moe_route_table_args {
+  uint32_t struct_size;
+  const int64_t* token_ids;    /* [num_tokens] */
+  const int32_t* table;        /* [vocab, top_k] */
+  int32_t* topk_ids;           /* out [num_tokens, top_k] */
+  float* topk_weights;         /* out [num_tokens, top_k] */
+  int32_t* expert_offsets;     /* out [num_experts + 1] */
+  int32_t* sorted_pair;        /* out [num_tokens * top_k] */
+  int32_t* pair_pos;           /* out [num_tokens * top_k] */
+  int32_t num_tokens, num_experts, top_k, vocab;
+} hymeta_moe_route_table_args;
+#define HYMETA_MOE_TABLE_MAX_EXPERTS 1024
+int hymeta_moe_route_table(const hymeta_moe_route_table_args* args, hymeta_stream_t stream);
+
+/* Grouped GEMM of the routed rows for any K and N and for fp32 or bf16 operands (hymeta_moe_gemm's
+ * tiles need K % 32 == 0, N % 64 == 0 and bf16): out[slot] = x[row(slot)] W[e]^T, fp32 sums.
+ * gated != 0: W[e] is [2 N, K] (gate rows, then up rows) and out[slot, n] = silu(gate_n) * up_n.
+ * row_scale as in hymeta_moe_gemm. */
+typedef struct hymeta_moe_gemm_any_args {
+  uint32_t struct_size;
+  const void* x;               /* act_dtype rows of K */
+  const void* weights;         /* act_dtype [experts, N (gated: 2 N), K] */
+  void* out;                   /* act_dtype [slots, N] */
+  const int32_t* expert_offsets;
+  const int32_t* a_rows;       /* source row of slot s = a_rows[s] / a_rows_div, or NULL: s */
+  const int32_t* scale_rows;   /* index into row_scale per slot, or NULL: s */
+  const float* row_scale;      /* or NULL */
+  int32_t a_rows_div, max_rows, K, N, num_experts, gated, act_dtype;
+  int64_t x_stride_m, out_stride_m, w_stride_e;
+} hymeta_moe_gemm_any_args;
+int hymeta_moe_gemm_any(const hymeta_moe_gemm_any_args* args, hymeta_stream_t stream);
+
+/* out[t] = sum_k y[pair_pos[t, k]] (rows with pair_pos < 0 are skipped), any width, fp32 or bf16. */
+typedef struct hymeta_moe_combine_any_args {
+  uint32_t struct_size;
+  const void* y;               /* act_dtype [slots, width] */
+  void* out;                   /* act_dtype [num_tokens, width] */
+  const int32_t* pair_pos;     /* [num_tokens, top_k] */
+  int32_t num_tokens, width, top_k, act_dtype;
+  int64_t y_stride_m, out_stride_m;
+} hymeta_moe_combine_any_args;
+int hymeta_moe_combine_any(const hymeta_moe_combine_any_args* args, hymeta_stream_t stream);
 
 #ifdef __cplusplus
 }

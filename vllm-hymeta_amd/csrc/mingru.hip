@@ -1,0 +1,107 @@
+// minGRU recurrence over a step's rows: per channel S <- (1 - z) S + z cand, out = S * silu(g), with the state
+// fp32 in registers and carried between steps in a slot-indexed tensor.
+//
+// The recurrence is linear in S (S' = a S + b with a = 1 - z, b = z cand), so a portion of a prompt is scanned in
+// parallel: a workgroup owns 64 channels of one sequence, its waves take consecutive runs of kRun rows, reduce each
+// run to its (product of a, value from zero), pass the carry over the waves through LDS and then replay their run
+// from the right starting state.  Sequences with one row (decode) run the one-wave form, which is the plain update.
+#include "act_types.h"
+
+namespace hymeta {
+
+namespace {
+
+constexpr int kRun = 8;              // rows per wave and round
+constexpr int kScanWaves = 8;        // waves of the prompt form
+
+template <typename A, int Waves>
+__global__ __launch_bounds__(64 * Waves) void mingru_kernel(hymeta_mingru_args a) {
+  typedef typename A::elem elem;
+  __shared__ float s_a[Waves][64], s_b[Waves][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int s = blockIdx.y;
+  const int c = blockIdx.x * 64 + lane;
+  const bool live = c < a.width;
+  const int64_t row0 = a.query_start_loc[s];
+  const int q = a.query_start_loc[s + 1] - static_cast<int>(row0);
+  if (q <= 0) return;
+  const int slot = a.slot_idx[s];
+  const int W = a.width;
+  float carry = 0.f;
+  if (live && slot >= 0 && a.context_lens[s] > 0) carry = a.state[static_cast<int64_t>(slot) * W + c];
+  const elem* zug = static_cast<const elem*>(a.zug);
+  elem* out = static_cast<elem*>(a.out);
+
+  for (int base = 0; base < q; base += kRun * Waves) {
+    const int lo = base + wave * kRun;
+    float av[kRun], bv[kRun], gv[kRun];
+#pragma unroll
+    for (int l = 0; l < kRun; ++l) {
+      av[l] = 1.f, bv[l] = 0.f, gv[l] = 0.f;
+      if (live && lo + l < q) {
+        const elem* r = zug + (row0 + lo + l) * a.zug_stride_t;
+        const float z = sigmoid_exact(A::ld(r + c));
+        const float u = A::ld(r + W + c);
+        const float cand = u >= 0.f ? u + 0.5f : sigmoid_exact(u);
+        const float g = A::ld(r + 2 * W + c);
+        av[l] = 1.f - z;
+        bv[l] = z * cand;
+        gv[l] = g * sigmoid_exact(g);
+      }
+    }
+    float S = carry;
+    if (Waves > 1) {
+      float pa = 1.f, pb = 0.f;
+#pragma unroll
+      for (int l = 0; l < kRun; ++l) {
+        pb = fmaf(av[l], pb, bv[l]);
+        pa *= av[l];
+      }
+      __syncthreads();                 // the round before has read the arrays
+      s_a[wave][lane] = pa;
+      s_b[wave][lane] = pb;
+      __syncthreads();
+      float next = carry;
+#pragma unroll
+      for (int w = 0; w < Waves; ++w) {
+        if (w == wave) S = next;
+        next = fmaf(s_a[w][lane], next, s_b[w][lane]);
+      }
+      carry = next;
+    }
+#pragma unroll
+    for (int l = 0; l < kRun; ++l) {
+      S = fmaf(av[l], S, bv[l]);
+      if (live && lo + l < q) A::st(out + (row0 + lo + l) * W + c, S * gv[l]);
+    }
+    if (Waves == 1) carry = S;
+  }
+  if (live && slot >= 0 && wave == 0) a.state[static_cast<int64_t>(slot) * W + c] = carry;
+}
+
+}  // namespace
+
+}  // namespace hymeta
+
+using namespace hymeta;
+
+extern "C" int hymeta_mingru(const hymeta_mingru_args* args, hymeta_stream_t stream) {
+  if (!args_ok(args)) return HYMETA_ERR_INVALID_ARG;
+  const hymeta_mingru_args& a = *args;
+  if (a.num_tokens < 0 || a.num_seqs < 0 || a.width <= 0) return HYMETA_ERR_INVALID_ARG;
+  if (!act_dtype_ok(a.act_dtype)) return HYMETA_ERR_UNSUPPORTED;
+  if (a.num_tokens == 0 || a.num_seqs == 0) return HYMETA_OK;
+  if (!a.zug || !a.state || !a.out || !a.query_start_loc || !a.context_lens || !a.slot_idx) return HYMETA_ERR_INVALID_ARG;
+  if (a.zug_stride_t < 3 * static_cast<int64_t>(a.width)) return HYMETA_ERR_INVALID_ARG;
+  const dim3 grid((a.width + 63) / 64, a.num_seqs);
+  hipStream_t st = begin_launches(stream);
+  const bool scan = a.max_query_len > kRun;
+  if (a.act_dtype == HYMETA_BF16) {
+    if (scan) hipLaunchKernelGGL((mingru_kernel<ActBf16, kScanWaves>), grid, dim3(64 * kScanWaves), 0, st, a);
+    else hipLaunchKernelGGL((mingru_kernel<ActBf16, 1>), grid, dim3(64), 0, st, a);
+  } else {
+    if (scan) hipLaunchKernelGGL((mingru_kernel<ActF32, kScanWaves>), grid, dim3(64 * kScanWaves), 0, st, a);
+    else hipLaunchKernelGGL((mingru_kernel<ActF32, 1>), grid, dim3(64), 0, st, a);
+  }
+  return launch_status();
+}

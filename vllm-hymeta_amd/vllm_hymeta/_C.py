@@ -24,7 +24,11 @@ GATE_7B = 1
 GATE_70B_CLAMP = 2
 GATE_70B_LOWER_BOUND = 3
 
-ABI_VERSION = 3
+BIAS_NONE = 0
+BIAS_LOG_DISTANCE = 1
+CONV_MAX_TAPS = 8
+
+ABI_VERSION = 4
 ERR_SCRATCH_LIMIT = -5
 GEMM_TICKET_BYTES = 16384
 STATIC_SCRATCH_BYTES = 16 << 20
@@ -285,6 +289,100 @@ class MoeCombineArgs(_Args):
 
 
 # symbol -> (restype, argtypes); every function include/hymeta_hip.h declares.
+
+
+class EmbedRowsArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("token_ids", _ptr), ("table", _ptr), ("add", _ptr), ("out", _ptr),
+        ("num_tokens", _i32), ("width", _i32), ("vocab", _i32), ("act_dtype", _i32),
+    ]
+
+
+class NormConvArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("x", _ptr), ("weight", _ptr), ("conv_weight", _ptr), ("conv_state", _ptr), ("out", _ptr),
+        ("query_start_loc", _ptr), ("context_lens", _ptr), ("slot_idx", _ptr),
+        ("num_tokens", _i32), ("num_seqs", _i32), ("width", _i32), ("taps", _i32), ("act_dtype", _i32),
+        ("eps", _f32), ("weight_offset", _f32),
+        ("x_stride_t", _i64),
+    ]
+
+
+class NormResidualArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("y", _ptr), ("weight", _ptr), ("post_add", _ptr), ("x", _ptr),
+        ("num_tokens", _i32), ("width", _i32), ("act_dtype", _i32),
+        ("eps", _f32), ("weight_offset", _f32), ("mult", _f32),
+        ("y_stride_t", _i64), ("x_stride_t", _i64),
+    ]
+
+
+class MinGruArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("zug", _ptr), ("state", _ptr), ("out", _ptr),
+        ("query_start_loc", _ptr), ("context_lens", _ptr), ("slot_idx", _ptr),
+        ("num_tokens", _i32), ("num_seqs", _i32), ("width", _i32), ("act_dtype", _i32), ("max_query_len", _i32),
+        ("zug_stride_t", _i64),
+    ]
+
+
+class QkNormCacheArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("qkv", _ptr), ("q_weight", _ptr), ("k_weight", _ptr), ("kv_cache", _ptr), ("slot_mapping", _ptr),
+        ("num_tokens", _i32), ("num_heads", _i32), ("num_kv_heads", _i32), ("head_dim", _i32), ("v_dim", _i32),
+        ("block_size", _i32), ("act_dtype", _i32),
+        ("eps", _f32),
+        ("num_blocks", _i64), ("qkv_stride_t", _i64),
+    ]
+
+
+class SinkAttentionArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("q", _ptr), ("kv_cache", _ptr), ("out", _ptr), ("block_tables", _ptr), ("query_start_loc", _ptr),
+        ("seq_lens", _ptr), ("bias_a", _ptr), ("bias_b", _ptr), ("workspace", _ptr), ("workspace_bytes", _sz),
+        ("num_tokens", _i32), ("num_seqs", _i32), ("num_heads", _i32), ("num_kv_heads", _i32), ("head_dim", _i32),
+        ("v_dim", _i32), ("block_size", _i32), ("act_dtype", _i32),
+        ("bias_mode", _i32), ("sink", _i32), ("window_left", _i32), ("max_query_len", _i32), ("max_seq_len", _i32),
+        ("scale", _f32),
+        ("num_blocks", _i64), ("q_stride_t", _i64), ("block_table_stride", _i64),
+    ]
+
+
+class MoeRouteTableArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("token_ids", _ptr), ("table", _ptr), ("topk_ids", _ptr), ("topk_weights", _ptr), ("expert_offsets", _ptr),
+        ("sorted_pair", _ptr), ("pair_pos", _ptr),
+        ("num_tokens", _i32), ("num_experts", _i32), ("top_k", _i32), ("vocab", _i32),
+    ]
+
+
+class MoeGemmAnyArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("x", _ptr), ("weights", _ptr), ("out", _ptr), ("expert_offsets", _ptr), ("a_rows", _ptr), ("scale_rows", _ptr),
+        ("row_scale", _ptr),
+        ("a_rows_div", _i32), ("max_rows", _i32), ("K", _i32), ("N", _i32), ("num_experts", _i32), ("gated", _i32),
+        ("act_dtype", _i32),
+        ("x_stride_m", _i64), ("out_stride_m", _i64), ("w_stride_e", _i64),
+    ]
+
+
+class MoeCombineAnyArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("y", _ptr), ("out", _ptr), ("pair_pos", _ptr),
+        ("num_tokens", _i32), ("width", _i32), ("top_k", _i32), ("act_dtype", _i32),
+        ("y_stride_m", _i64), ("out_stride_m", _i64),
+    ]
+
+
 _SIGNATURES = {
     "hymeta_strerror": (C.c_char_p, [C.c_int]),
     "hymeta_abi_version": (C.c_int, []),
@@ -352,6 +450,16 @@ _SIGNATURES = {
     "hymeta_w8a8_scale_out": (C.c_int, [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _i32, _i64, _i64, _ptr]),
     "hymeta_w8a8_gemm_split_k": (C.c_int, [_i32, _i32, _i32]),
     "hymeta_w8a8_gemm_workspace_bytes": (_sz, [_i32, _i32, _i32]),
+    "hymeta_embed_rows": (C.c_int, [C.POINTER(EmbedRowsArgs), _ptr]),
+    "hymeta_norm_conv": (C.c_int, [C.POINTER(NormConvArgs), _ptr]),
+    "hymeta_norm_residual": (C.c_int, [C.POINTER(NormResidualArgs), _ptr]),
+    "hymeta_mingru": (C.c_int, [C.POINTER(MinGruArgs), _ptr]),
+    "hymeta_qk_norm_cache": (C.c_int, [C.POINTER(QkNormCacheArgs), _ptr]),
+    "hymeta_sink_attention_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32]),
+    "hymeta_sink_attention": (C.c_int, [C.POINTER(SinkAttentionArgs), _ptr]),
+    "hymeta_moe_route_table": (C.c_int, [C.POINTER(MoeRouteTableArgs), _ptr]),
+    "hymeta_moe_gemm_any": (C.c_int, [C.POINTER(MoeGemmAnyArgs), _ptr]),
+    "hymeta_moe_combine_any": (C.c_int, [C.POINTER(MoeCombineAnyArgs), _ptr]),
 }
 
 STRUCTS = {
@@ -373,6 +481,15 @@ STRUCTS = {
     "hymeta_moe_gemm_args": MoeGemmArgs,
     "hymeta_moe_gptq_gemm_args": MoeGptqGemmArgs,
     "hymeta_moe_combine_args": MoeCombineArgs,
+    "hymeta_embed_rows_args": EmbedRowsArgs,
+    "hymeta_norm_conv_args": NormConvArgs,
+    "hymeta_norm_residual_args": NormResidualArgs,
+    "hymeta_mingru_args": MinGruArgs,
+    "hymeta_qk_norm_cache_args": QkNormCacheArgs,
+    "hymeta_sink_attention_args": SinkAttentionArgs,
+    "hymeta_moe_route_table_args": MoeRouteTableArgs,
+    "hymeta_moe_gemm_any_args": MoeGemmAnyArgs,
+    "hymeta_moe_combine_any_args": MoeCombineAnyArgs,
 }
 
 

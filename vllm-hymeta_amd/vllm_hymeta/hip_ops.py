@@ -1457,3 +1457,257 @@ def moe_forward(x: torch.Tensor, router_logits: Optional[torch.Tensor], w13: tor
         c.shared_stride_m = shared.stride(0)
     _C.check(lib.hymeta_moe_combine(C.byref(c), st), "hymeta_moe_combine")
     return out
+
+
+# ---------------------------------------------------------------------------
+# Building blocks of recurrent / biased-attention designs: fp32 residual stream, norm + short convolution,
+# minGRU, paged attention with a distance bias and a sink, table-routed experts.  Activations bf16 or fp32.
+# ---------------------------------------------------------------------------
+def _act(t: torch.Tensor) -> int:
+    _require(t.dtype in _DT, "activations must be bf16 or fp32")
+    return _DT[t.dtype]
+
+
+def _f32vec(t: Optional[torch.Tensor], n: int, name: str) -> None:
+    _require(t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n), f"{name} must be contiguous fp32 [{n}]")
+
+
+def _i32vec(t: torch.Tensor, n: int, name: str) -> None:
+    _require(t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= n, f"{name} must be contiguous int32 [{n}]")
+
+
+def embed_rows(token_ids: torch.Tensor, table: torch.Tensor, add: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 ``[T, W]`` rows ``table[token_ids] (+ add)``: the start of an fp32 residual stream."""
+    _dev(token_ids, table, add)
+    _require(token_ids.dtype == torch.int64 and token_ids.dim() == 1 and token_ids.is_contiguous(), "token_ids must be contiguous int64 [T]")
+    _require(table.dim() == 2 and table.is_contiguous(), "table must be contiguous [vocab, width]")
+    V, W = table.shape
+    _f32vec(add, W, "add")
+    out = torch.empty(token_ids.shape[0], W, dtype=torch.float32, device=table.device)
+    a = _C.EmbedRowsArgs()
+    a.token_ids, a.table, a.add, a.out = _p(token_ids), _p(table), _p(add), _p(out)
+    a.num_tokens, a.width, a.vocab, a.act_dtype = token_ids.shape[0], W, V, _act(table)
+    _C.check(_C.load().hymeta_embed_rows(C.byref(a), _stream(table)), "hymeta_embed_rows")
+    return out
+
+
+def norm_conv(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype, weight_offset: float = 0.0,
+              conv_weight: Optional[torch.Tensor] = None, conv_state: Optional[torch.Tensor] = None,
+              query_start_loc: Optional[torch.Tensor] = None, context_lens: Optional[torch.Tensor] = None,
+              slot_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMS norm of the fp32 rows ``x [T, W]`` (weight ``weight_offset + weight``), then, with ``conv_weight [W, taps]``,
+    ``out[t] = n[t] + sum_j conv_weight[:, j] n[t - taps + 1 + j]`` over each sequence's rows; ``conv_state
+    [slots, taps - 1, W]`` (``out_dtype``) carries a sequence's last rows between steps and is updated in place."""
+    _dev(x, weight, conv_weight, conv_state, query_start_loc, context_lens, slot_idx)
+    _require(x.dim() == 2 and x.dtype == torch.float32 and x.stride(1) == 1, "x must be row-contiguous fp32 [T, W]")
+    T, W = x.shape
+    _f32vec(weight, W, "weight")
+    _require(out_dtype in _DT, "out_dtype must be bf16 or fp32")
+    out = torch.empty(T, W, dtype=out_dtype, device=x.device)
+    a = _C.NormConvArgs()
+    a.x, a.weight, a.out = _p(x), _p(weight), _p(out)
+    a.num_tokens, a.width, a.act_dtype, a.eps, a.weight_offset, a.x_stride_t = T, W, _DT[out_dtype], eps, weight_offset, x.stride(0)
+    a.taps = 1
+    if conv_weight is not None:
+        taps = conv_weight.shape[1]
+        _require(conv_weight.dtype == torch.float32 and conv_weight.is_contiguous() and conv_weight.shape == (W, taps),
+                 "conv_weight must be contiguous fp32 [W, taps]")
+        _require(1 <= taps <= _C.CONV_MAX_TAPS, f"taps must be 1 .. {_C.CONV_MAX_TAPS}")
+        a.conv_weight, a.taps = _p(conv_weight), taps
+        if taps > 1:
+            _require(query_start_loc is not None and context_lens is not None, "a convolution over time needs the step's sequence layout")
+            S = query_start_loc.numel() - 1
+            _i32vec(query_start_loc, S + 1, "query_start_loc")
+            _i32vec(context_lens, S, "context_lens")
+            a.query_start_loc, a.context_lens, a.num_seqs = _p(query_start_loc), _p(context_lens), S
+            if conv_state is not None:
+                _require(slot_idx is not None, "conv_state needs slot_idx")
+                _i32vec(slot_idx, S, "slot_idx")
+                _require(conv_state.dtype == out_dtype and conv_state.is_contiguous() and conv_state.dim() == 3
+                         and conv_state.shape[1:] == (taps - 1, W), "conv_state must be contiguous [slots, taps - 1, W] of out_dtype")
+                a.conv_state, a.slot_idx = _p(conv_state), _p(slot_idx)
+    _C.check(_C.load().hymeta_norm_conv(C.byref(a), _stream(x)), "hymeta_norm_conv")
+    return out
+
+
+def norm_residual_(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float, mult: float = 1.0,
+                   weight_offset: float = 0.0, post_add: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x += mult * rmsnorm(y) * (weight_offset + weight) (+ post_add)`` on the fp32 rows ``x [T, W]``, in place."""
+    _dev(x, y, weight, post_add)
+    _require(x.dim() == 2 and x.dtype == torch.float32 and x.stride(1) == 1, "x must be row-contiguous fp32 [T, W]")
+    T, W = x.shape
+    _require(y.shape == (T, W) and y.stride(1) == 1, "y must be row-contiguous [T, W]")
+    _f32vec(weight, W, "weight")
+    _f32vec(post_add, W, "post_add")
+    a = _C.NormResidualArgs()
+    a.y, a.weight, a.post_add, a.x = _p(y), _p(weight), _p(post_add), _p(x)
+    a.num_tokens, a.width, a.act_dtype = T, W, _act(y)
+    a.eps, a.weight_offset, a.mult, a.y_stride_t, a.x_stride_t = eps, weight_offset, mult, y.stride(0), x.stride(0)
+    _C.check(_C.load().hymeta_norm_residual(C.byref(a), _stream(x)), "hymeta_norm_residual")
+    return x
+
+
+def mingru(zug: torch.Tensor, state: torch.Tensor, query_start_loc: torch.Tensor, context_lens: torch.Tensor,
+           slot_idx: torch.Tensor, max_query_len: int) -> torch.Tensor:
+    """minGRU over a step's rows: ``zug [T, 3W]`` = the update-gate, candidate and output-gate projections;
+    ``state`` fp32 ``[slots, W]`` is read (where ``context_lens > 0``) and written.  Returns ``S * silu(g)`` ``[T, W]``."""
+    _dev(zug, state, query_start_loc, context_lens, slot_idx)
+    _require(zug.dim() == 2 and zug.stride(1) == 1 and zug.shape[1] % 3 == 0, "zug must be row-contiguous [T, 3W]")
+    T, W = zug.shape[0], zug.shape[1] // 3
+    _require(state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 2 and state.shape[1] == W, "state must be contiguous fp32 [slots, W]")
+    S = query_start_loc.numel() - 1
+    _i32vec(query_start_loc, S + 1, "query_start_loc")
+    _i32vec(context_lens, S, "context_lens")
+    _i32vec(slot_idx, S, "slot_idx")
+    out = torch.empty(T, W, dtype=zug.dtype, device=zug.device)
+    a = _C.MinGruArgs()
+    a.zug, a.state, a.out = _p(zug), _p(state), _p(out)
+    a.query_start_loc, a.context_lens, a.slot_idx = _p(query_start_loc), _p(context_lens), _p(slot_idx)
+    a.num_tokens, a.num_seqs, a.width, a.act_dtype, a.max_query_len, a.zug_stride_t = T, S, W, _act(zug), max_query_len, zug.stride(0)
+    _C.check(_C.load().hymeta_mingru(C.byref(a), _stream(zug)), "hymeta_mingru")
+    return out
+
+
+def qk_norm_cache_(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, v_dim: int,
+                   q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                   kv_cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor]) -> None:
+    """Per-head RMS norm of the query / key columns of ``qkv [T, H D + G D + G Dv]`` (queries in place) and the paged
+    write of the normed keys and the values into ``kv_cache [blocks, block_size, G, D + Dv]`` at ``slot_mapping``."""
+    _dev(qkv, q_weight, k_weight, kv_cache, slot_mapping)
+    T = qkv.shape[0]
+    _require(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim,
+             "qkv must be row-contiguous [T, H D + G D + G Dv]")
+    _f32vec(q_weight, head_dim, "q_weight")
+    _f32vec(k_weight, head_dim, "k_weight")
+    a = _C.QkNormCacheArgs()
+    a.qkv, a.q_weight, a.k_weight = _p(qkv), _p(q_weight), _p(k_weight)
+    a.num_tokens, a.num_heads, a.num_kv_heads, a.head_dim, a.v_dim = T, num_heads, num_kv_heads, head_dim, v_dim
+    a.act_dtype, a.eps, a.qkv_stride_t, a.block_size = _act(qkv), eps, qkv.stride(0), 1
+    if kv_cache is not None and kv_cache.numel() > 0 and slot_mapping is not None:
+        _require(kv_cache.dtype == qkv.dtype and kv_cache.is_contiguous() and kv_cache.dim() == 4
+                 and kv_cache.shape[2:] == (num_kv_heads, head_dim + v_dim), "kv_cache must be contiguous [blocks, block_size, G, D + Dv]")
+        _require(slot_mapping.dtype == torch.int64 and slot_mapping.is_contiguous() and slot_mapping.numel() == T, "slot_mapping must be int64 [T]")
+        a.kv_cache, a.slot_mapping, a.num_blocks, a.block_size = _p(kv_cache), _p(slot_mapping), kv_cache.shape[0], kv_cache.shape[1]
+    _C.check(_C.load().hymeta_qk_norm_cache(C.byref(a), _stream(qkv)), "hymeta_qk_norm_cache")
+
+
+def sink_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_tables: torch.Tensor, query_start_loc: torch.Tensor,
+                   seq_lens: torch.Tensor, num_kv_heads: int, head_dim: int, v_dim: int, scale: float,
+                   max_query_len: int, max_seq_len: int, bias_a: Optional[torch.Tensor] = None,
+                   bias_b: Optional[torch.Tensor] = None, sink: bool = True, window_left: int = -1) -> torch.Tensor:
+    """Causal attention of the rows ``q [T, H, D]`` over their sequences' paged keys (this step's included):
+    ``softmax`` over ``scale q.k - bias_a[h] ln(1 + bias_b[h] (i - j))`` with, for ``sink``, one added to the denominator.
+    Returns ``[T, H, Dv]``."""
+    _dev(q, kv_cache, block_tables, query_start_loc, seq_lens, bias_a, bias_b)
+    _require(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == head_dim and q.shape[2] == head_dim, "q must be [T, H, D] with contiguous heads")
+    T, H, _ = q.shape
+    _require(kv_cache.dtype == q.dtype and kv_cache.is_contiguous() and kv_cache.dim() == 4
+             and kv_cache.shape[2:] == (num_kv_heads, head_dim + v_dim), "kv_cache must be contiguous [blocks, block_size, G, D + Dv]")
+    S = query_start_loc.numel() - 1
+    _i32vec(query_start_loc, S + 1, "query_start_loc")
+    _i32vec(seq_lens, S, "seq_lens")
+    _require(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.shape[0] >= S and block_tables.stride(1) == 1,
+             "block_tables must be int32 [S, blocks]")
+    _require((bias_a is None) == (bias_b is None), "bias_a and bias_b come together")
+    _f32vec(bias_a, H, "bias_a")
+    _f32vec(bias_b, H, "bias_b")
+    out = torch.empty(T, H, v_dim, dtype=q.dtype, device=q.device)
+    lib = _C.load()
+    a = _C.SinkAttentionArgs()
+    a.q, a.kv_cache, a.out, a.block_tables = _p(q), _p(kv_cache), _p(out), _p(block_tables)
+    a.query_start_loc, a.seq_lens, a.bias_a, a.bias_b = _p(query_start_loc), _p(seq_lens), _p(bias_a), _p(bias_b)
+    nbytes = int(lib.hymeta_sink_attention_workspace_bytes(T, H, v_dim, max_seq_len))
+    if nbytes:
+        ws = _workspace(q.device, nbytes, "sink_attention")
+        a.workspace, a.workspace_bytes = _p(ws), ws.numel()
+    a.num_tokens, a.num_seqs, a.num_heads, a.num_kv_heads, a.head_dim, a.v_dim = T, S, H, num_kv_heads, head_dim, v_dim
+    a.block_size, a.act_dtype, a.num_blocks = kv_cache.shape[1], _act(q), kv_cache.shape[0]
+    a.bias_mode = _C.BIAS_NONE if bias_a is None else _C.BIAS_LOG_DISTANCE
+    a.sink, a.window_left, a.max_query_len, a.max_seq_len, a.scale = int(bool(sink)), window_left, max_query_len, max_seq_len, scale
+    a.q_stride_t, a.block_table_stride = q.stride(0), block_tables.stride(0)
+    _C.check(lib.hymeta_sink_attention(C.byref(a), _stream(q)), "hymeta_sink_attention")
+    return out
+
+
+def moe_mfma_shapes(hidden: int, inter: int) -> bool:
+    """Whether the routed block's MFMA grouped GEMMs take experts of these sizes (bf16: K in whole 32s, N in whole 64s)."""
+    return hidden % 64 == 0 and inter % 32 == 0 and (2 * inter) % 64 == 0
+
+
+def moe_table_forward(x: torch.Tensor, token_ids: torch.Tensor, table: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor) -> torch.Tensor:
+    """Experts chosen by ``table[token_id]`` (int32 ``[vocab, top]``), each weighing ``1 / top``: ``x [T, H]``, ``w13
+    [E, 2I, H]`` (gate rows, then up rows), ``w2 [E, H, I]``, all bf16 or all fp32.  The counting sort by expert is
+    one launch; bf16 experts in the MFMA tiles' shapes then run the routed block's grouped GEMMs, activation and
+    combine, everything else the generic grouped GEMM (activation in its epilogue) and combine."""
+    _dev(x, token_ids, table, w13, w2)
+    T, H = x.shape
+    E, two_i, _ = w13.shape
+    inter = two_i // 2
+    top = table.shape[1]
+    _require(x.dtype in _DT and x.stride(1) == 1 and w13.dtype == x.dtype and w2.dtype == x.dtype, "x, w13 and w2 must share bf16 or fp32")
+    _require(w13.is_contiguous() and w13.shape == (E, 2 * inter, H) and w2.is_contiguous() and w2.shape == (E, H, inter),
+             "w13 must be contiguous [E, 2I, H] and w2 [E, H, I]")
+    _require(table.dtype == torch.int32 and table.is_contiguous() and table.dim() == 2, "table must be contiguous int32 [vocab, top]")
+    _require(token_ids.dtype == torch.int64 and token_ids.is_contiguous() and token_ids.numel() == T, "token_ids must be contiguous int64 [T]")
+    dev = x.device
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    if T == 0:
+        return out
+    P = T * top
+    ids = torch.empty(T, top, dtype=torch.int32, device=dev)
+    wts = torch.empty(T, top, dtype=torch.float32, device=dev)
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    sorted_pair = torch.empty(P, dtype=torch.int32, device=dev)
+    pair_pos = torch.empty(P, dtype=torch.int32, device=dev)
+    lib, st = _C.load(), _stream(x)
+    r = _C.MoeRouteTableArgs()
+    r.token_ids, r.table, r.topk_ids, r.topk_weights = _p(token_ids), _p(table), _p(ids), _p(wts)
+    r.expert_offsets, r.sorted_pair, r.pair_pos = _p(offsets), _p(sorted_pair), _p(pair_pos)
+    r.num_tokens, r.num_experts, r.top_k, r.vocab = T, E, top, table.shape[0]
+    _C.check(lib.hymeta_moe_route_table(C.byref(r), st), "hymeta_moe_route_table")
+
+    if (x.dtype == torch.bfloat16 and moe_mfma_shapes(H, inter) and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
+        h13 = torch.empty(P, two_i, dtype=torch.bfloat16, device=dev)
+        g = _C.MoeGemmArgs()
+        g.x, g.weights, g.out, g.expert_offsets = _p(x), _p(w13), _p(h13), _p(offsets)
+        g.a_rows, g.a_rows_div, g.max_rows, g.K, g.N = _p(sorted_pair), top, P, H, two_i
+        g.local_expert_begin, g.local_expert_end = 0, E
+        g.x_stride_m, g.out_stride_m, g.w_stride_e = x.stride(0), h13.stride(0), w13.stride(0)
+        _C.check(lib.hymeta_moe_gemm(C.byref(g), st), "hymeta_moe_gemm (w13)")
+        hact = torch.empty(P, inter, dtype=torch.bfloat16, device=dev)
+        silu_and_mul(h13, out=hact)
+        y = torch.empty(P, H, dtype=torch.bfloat16, device=dev)
+        d = _C.MoeGemmArgs()
+        d.x, d.x_stride_m, d.weights, d.out, d.expert_offsets = _p(hact), hact.stride(0), _p(w2), _p(y), _p(offsets)
+        d.scale_rows, d.row_scale = _p(sorted_pair), _p(wts)
+        d.a_rows_div, d.max_rows, d.K, d.N = 1, P, inter, H
+        d.local_expert_begin, d.local_expert_end = 0, E
+        d.out_stride_m, d.w_stride_e = y.stride(0), w2.stride(0)
+        _C.check(lib.hymeta_moe_gemm(C.byref(d), st), "hymeta_moe_gemm (w2)")
+        c = _C.MoeCombineArgs()
+        c.y, c.out, c.pair_pos, c.topk_weights = _p(y), _p(out), _p(pair_pos), _p(wts)
+        c.num_tokens, c.hidden, c.top_k = T, H, top
+        c.y_stride_m, c.out_stride_m = y.stride(0), out.stride(0)
+        _C.check(lib.hymeta_moe_combine(C.byref(c), st), "hymeta_moe_combine")
+        return out
+
+    act = _DT[x.dtype]
+    hact = torch.empty(P, inter, dtype=x.dtype, device=dev)
+    g = _C.MoeGemmAnyArgs()
+    g.x, g.weights, g.out, g.expert_offsets = _p(x), _p(w13), _p(hact), _p(offsets)
+    g.a_rows, g.a_rows_div, g.max_rows, g.K, g.N, g.num_experts, g.gated, g.act_dtype = _p(sorted_pair), top, P, H, inter, E, 1, act
+    g.x_stride_m, g.out_stride_m, g.w_stride_e = x.stride(0), hact.stride(0), w13.stride(0)
+    _C.check(lib.hymeta_moe_gemm_any(C.byref(g), st), "hymeta_moe_gemm_any (w13)")
+    y = torch.empty(P, H, dtype=x.dtype, device=dev)
+    d = _C.MoeGemmAnyArgs()
+    d.x, d.weights, d.out, d.expert_offsets = _p(hact), _p(w2), _p(y), _p(offsets)
+    d.scale_rows, d.row_scale = _p(sorted_pair), _p(wts)
+    d.a_rows_div, d.max_rows, d.K, d.N, d.num_experts, d.gated, d.act_dtype = 1, P, inter, H, E, 0, act
+    d.x_stride_m, d.out_stride_m, d.w_stride_e = hact.stride(0), y.stride(0), w2.stride(0)
+    _C.check(lib.hymeta_moe_gemm_any(C.byref(d), st), "hymeta_moe_gemm_any (w2)")
+    c = _C.MoeCombineAnyArgs()
+    c.y, c.out, c.pair_pos = _p(y), _p(out), _p(pair_pos)
+    c.num_tokens, c.width, c.top_k, c.act_dtype = T, H, top, act
+    c.y_stride_m, c.out_stride_m = y.stride(0), out.stride(0)
+    _C.check(lib.hymeta_moe_combine_any(C.byref(c), st), "hymeta_moe_combine_any")
+    return out

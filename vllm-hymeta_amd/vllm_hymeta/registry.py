@@ -1,0 +1,54 @@
+"""Which model class and configuration class serve which ``config.json``: the table behind the vLLM registration hooks
+(``register_model``) and behind the package's own engine, which has no vLLM to ask."""
+
+from __future__ import annotations
+
+import importlib
+import json
+import os
+from typing import Any, Callable, Dict, Tuple
+
+# architecture name (``architectures[0]`` or ``architecture`` of config.json) -> (module:class of the model, loader of its config)
+_MODELS: Dict[str, Tuple[str, Callable[[str], Any]]] = {}
+
+
+def register(architecture: str, model_path: str, config_loader: Callable[[str], Any]) -> None:
+    _MODELS[architecture] = (model_path, config_loader)
+
+
+def _sonuzen_config(model_dir: str):
+    from .models.configuration_sonuzen import SonuzenConfig
+    return SonuzenConfig.from_pretrained(model_dir)
+
+
+def _gla_swa_config(model_dir: str):
+    from .model_for_7B.configuration_gla_swa import GLAswaConfig
+    with open(os.path.join(model_dir, "config.json")) as f:
+        raw = json.load(f)
+    raw.pop("architectures", None), raw.pop("model_type", None)
+    return GLAswaConfig(**raw)
+
+
+register("Sonuzen", "vllm_hymeta.models.modeling_sonuzen:SonuzenForCausalLM", _sonuzen_config)
+register("SonuzenForCausalLM", "vllm_hymeta.models.modeling_sonuzen:SonuzenForCausalLM", _sonuzen_config)
+register("GLAswaForCausalLM", "vllm_hymeta.model_for_7B.modeling_gla_swa:GLAswaForCausalLM", _gla_swa_config)
+
+
+def architecture_of(model_dir: str) -> str:
+    with open(os.path.join(model_dir, "config.json")) as f:
+        raw = json.load(f)
+    arch = raw.get("architecture") or (raw.get("architectures") or [None])[0]
+    if arch not in _MODELS:
+        raise ValueError(f"{model_dir}: architecture {arch!r} is not served by this package (known: {sorted(_MODELS)})")
+    return arch
+
+
+def resolve(model_dir: str):
+    """``(model class, config)`` for a checkpoint folder."""
+    path, load_config = _MODELS[architecture_of(model_dir)]
+    module, _, name = path.partition(":")
+    return getattr(importlib.import_module(module), name), load_config(model_dir)
+
+
+def known_architectures():
+    return sorted(_MODELS)
