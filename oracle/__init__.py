@@ -38,3 +38,14 @@ from .paged import (  # noqa: F401
     gather_paged_ref,
     kv_cache_shape_ref,
 )
+from .sonuzen import (  # noqa: F401
+    attention_mixer_ref,
+    causal_conv_add_ref,
+    mingru_ref,
+    norm_one_plus_ref,
+    sink_attention_ref,
+    sonuzen_config,
+    sonuzen_random_weights,
+    sonuzen_ref,
+    table_moe_ref,
+)

@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kNormThreads) void norm_conv_kernel(hymeta_norm_con
       const float w = a.weight_offset + a.weight[c];
       const float n = A::round(a.x[(row0 + ii) * a.x_stride_t + c] * inv[hist] * w);
       float acc = n;
-      if (hist > 0) {
+      if (a.conv_weight != nullptr) {
         const float* cw = a.conv_weight + static_cast<int64_t>(c) * taps;
         acc = fmaf(cw[hist], n, acc);
         for (int j = 0; j < hist; ++j) {

@@ -41,6 +41,7 @@ class Request:
     num_computed: int = 0                             # tokens whose keys / states are in the caches
     blocks: List[int] = field(default_factory=list)
     finished: bool = False
+    state_key: str = ""                               # the name the model's state cache knows the request by
 
     @property
     def output_token_ids(self) -> List[int]:
@@ -129,6 +130,7 @@ class LLMEngine:
         self.requests: Dict[str, Request] = {}
         self._finished_since_last_step: List[str] = []
         self._generators: Dict[str, torch.Generator] = {}
+        self._serial = 0
         prefix = getattr(getattr(model, "model", model), "prefix", None)
         if prefix is None:
             raise ValueError("the model does not say under which prefix its attention layers are registered")
@@ -168,6 +170,9 @@ class LLMEngine:
         if request_id in self.requests:
             raise ValueError(f"request {request_id!r} is live already")
         r = Request(request_id, list(prompt_token_ids), len(prompt_token_ids), params or SamplingParams())
+        # a name of its own for the state cache: a request id that comes back after its first owner ended is a new request
+        self._serial += 1
+        r.state_key = f"{request_id}#{self._serial}"
         self.requests[request_id] = r
         if schedule:
             self.scheduler.add(r)
@@ -180,7 +185,7 @@ class LLMEngine:
         r.finished = True
         self.pool.release(r.blocks)
         self.scheduler.retire(r)
-        self._finished_since_last_step.append(request_id)
+        self._finished_since_last_step.append(r.state_key)
         self._generators.pop(request_id, None)
 
     # ------------------------------------------------------------------ the step function
@@ -215,7 +220,7 @@ class LLMEngine:
             positions.extend(range(ctx, ctx + n))
             slot_mapping.extend(r.blocks[p // bs] * bs + p % bs for p in range(ctx, ctx + n))
             query_lens.append(n), seq_lens.append(ctx + n), context_lens.append(ctx), tables.append(list(r.blocks))
-            ids[r.request_id] = [0]
+            ids[r.state_key] = [0]
             if not (n == 1 and ctx > 0):
                 num_prefills += 1
                 num_prefill_tokens += n

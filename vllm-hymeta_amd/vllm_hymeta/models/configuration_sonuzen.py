@@ -53,7 +53,8 @@ class SonuzenConfig:
         self.norm_eps = float(raw["norm"]["eps"])
         self.residual_mult = float(raw.get("residual_mult", 1.0))
         self.logit_scale = float(raw.get("logit_scale", 1.0))
-        self.conv_taps = int((raw.get("canon") or {}).get("taps", 1))
+        self.has_conv = bool(raw.get("canon"))
+        self.conv_taps = int(raw["canon"]["taps"]) if self.has_conv else 1
         self.layers: List[SonuzenLayerSpec] = []
         for i, entry in enumerate(raw["layers"]):
             kind, mx = entry["type"], entry.get("mixer") or {}

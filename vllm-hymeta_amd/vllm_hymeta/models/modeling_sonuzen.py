@@ -30,17 +30,21 @@ from .table_moe import TableMoE
 
 
 class SonuzenStateCache(ConstantSizeStateCache):
-    """``recurrent [R, slots, W]`` fp32: one minGRU state per (minGRU layer, pass); ``conv [C, slots, taps - 1, W]`` in the
-    activation type: the last inputs of every sublayer's convolution, per (layer, pass, sublayer)."""
+    """``recurrent[r] [1, slots, width_r]`` fp32: the minGRU state of the ``r``-th (minGRU layer, pass); ``conv
+    [C, slots, taps - 1, W]`` in the activation type: the last inputs of every sublayer's convolution, per (layer, pass,
+    sublayer)."""
 
-    def __init__(self, num_recurrent: int, num_conv: int, max_batch_size: int, width: int, history: int, dtype, device):
+    def __init__(self, recurrent_widths: List[int], num_conv: int, max_batch_size: int, width: int, history: int, dtype, device):
         super().__init__(max_batch_size, device)
-        self.recurrent = torch.zeros(max(num_recurrent, 1), max_batch_size, width, dtype=torch.float32, device=self.device)
+        self.recurrent = [torch.zeros(1, max_batch_size, w, dtype=torch.float32, device=self.device) for w in recurrent_widths]
         self.conv = torch.zeros(max(num_conv, 1), max_batch_size, max(history, 1), width, dtype=dtype, device=self.device)
 
     @property
     def cache(self):
         return (self.recurrent, self.conv)
+
+    def _slot_tensors(self):
+        return tuple(self.recurrent) + (self.conv,)
 
 
 class SonuzenModel(torch.nn.Module):
@@ -66,17 +70,15 @@ class SonuzenModel(torch.nn.Module):
                                                            f"{self.prefix}.layers.{i}.pass{t}.attn", dtype=dtype)
                 self._attn_key[(i, t)] = key
             else:
-                if spec.mixer.width != config.hidden_size:
-                    raise ValueError("a minGRU mixer is as wide as the model")
                 self._recurrent_index[(i, t)] = len(self._recurrent_index)
-        self.history = max(config.conv_taps - 1, 0)
+        self.history = max(config.conv_taps - 1, 0) if config.has_conv else 0
         self._conv_index: Dict[Tuple[int, int], int] = {}
         n_conv = 0
         for (i, t) in self.runs:
             self._conv_index[(i, t)] = n_conv
             n_conv += (1 + int(config.layers[i].mlp is not None)) if self.history else 0
-        self.state_cache = SonuzenStateCache(len(self._recurrent_index), n_conv, max_num_seqs, config.hidden_size, self.history,
-                                             dtype, self.device)
+        widths = [config.layers[i].mixer.width for (i, t) in self.runs if (i, t) in self._recurrent_index]
+        self.state_cache = SonuzenStateCache(widths, n_conv, max_num_seqs, config.hidden_size, self.history, dtype, self.device)
         self.embed: Optional[torch.Tensor] = None
         self.loop_step: Optional[torch.Tensor] = None        # fp32 [times, W]
         self.layers = torch.nn.ModuleList()
@@ -124,7 +126,7 @@ class SonuzenModel(torch.nn.Module):
             if (i, t) in self._attn_key:
                 mixer_state = self.attn_layers[self._attn_key[(i, t)]]
             else:
-                mixer_state = recurrent[self._recurrent_index[(i, t)]]
+                mixer_state = recurrent[self._recurrent_index[(i, t)]][0]
             c0 = self._conv_index[(i, t)]
             x = block(x, self.dtype, layout, mixer_state, [conv[c0 + j] for j in range(block.conv_states)], self._post_add(n))
             if residual_out is not None:
@@ -210,7 +212,7 @@ class SonuzenForCausalLM(torch.nn.Module, HasInnerState, IsHybrid):
             if m.loop_step.shape != (cfg.loop_times, W):
                 raise ValueError(f"loop.step is {tuple(m.loop_step.shape)}, the loop runs {cfg.loop_times} times over width {W}")
         m.layers = torch.nn.ModuleList()
-        conv = cfg.conv_taps > 1
+        conv = cfg.has_conv
         for i, spec in enumerate(cfg.layers):
             p = f"l{i}."
             if spec.type == "attention":
@@ -228,7 +230,9 @@ class SonuzenForCausalLM(torch.nn.Module, HasInnerState, IsHybrid):
                     raise ValueError(f"layer {i}: attention projections do not have the configured sizes")
             else:
                 mixer = MinGRUMixer(linear([p + "mix.z", p + "mix.x", p + "mix.g"], [p + "mix.z.b", p + "mix.x.b", None]),
-                                    linear([p + "mix.o"]), W)
+                                    linear([p + "mix.o"]), spec.mixer.width)
+                if tuple(mixer.zug_proj.weight.shape) != (3 * spec.mixer.width, W) or tuple(mixer.o_proj.weight.shape) != (W, spec.mixer.width):
+                    raise ValueError(f"layer {i}: minGRU projections do not have the configured sizes")
             mixer_in = NormConvIn(f32(p + "norm1"), cfg.norm_eps, f32(p + "canon1") if conv else None)
             mixer_out = NormOutResidual(f32(p + "norm1b"), cfg.norm_eps, cfg.residual_mult)
             mlp_in = mlp = mlp_out = None
