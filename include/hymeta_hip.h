@@ -1161,9 +1161,12 @@ int hymeta_qk_norm_cache(const hymeta_qk_norm_cache_args* args, hymeta_stream_t 
  *   p_ij = exp(s_ij) / (sink + sum_j exp(s_ij)),  sink = 1 (a key of score 0 without a value) or 0
  *   out_i = sum_j p_ij v_j
  * Scores and weights are fp32 in both activation types.  Query row t of sequence s stands at position
- * seq_lens[s] - (query_start_loc[s + 1] - t).  Sequences with one query row (decode) and portions of
- * prompts run in the same launch sequence; `workspace` (hymeta_sink_attention_workspace_bytes) holds
- * the partial results of long single-row sequences split over their keys. */
+ * seq_lens[s] - (query_start_loc[s + 1] - t).  bf16 rows with head_dim and v_dim of 64 or 128 (and at
+ * most 32 query heads per key/value head) run on the matrix cores: portions of prompts in tiles of 128
+ * rows, sequences with one row (decode) per key/value head with all its query heads, split over the
+ * keys into `workspace` (hymeta_sink_attention_workspace_bytes) and merged by a second launch.
+ * max_query_len / max_seq_len: upper bounds of the step's portion and sequence lengths (they size the
+ * grids).  Everything else runs a wave per (row, head). */
 enum hymeta_bias_mode { HYMETA_BIAS_NONE = 0, HYMETA_BIAS_LOG_DISTANCE = 1 };
 typedef struct hymeta_sink_attention_args {
   uint32_t struct_size;
@@ -1182,7 +1185,8 @@ typedef struct hymeta_sink_attention_args {
   float scale;
   int64_t num_blocks, q_stride_t, block_table_stride;
 } hymeta_sink_attention_args;
-size_t hymeta_sink_attention_workspace_bytes(int32_t num_tokens, int32_t num_heads, int32_t v_dim, int32_t max_seq_len);
+size_t hymeta_sink_attention_workspace_bytes(int32_t num_seqs, int32_t num_heads, int32_t num_kv_heads, int32_t v_dim,
+                                             int32_t max_seq_len);
 int hymeta_sink_attention(const hymeta_sink_attention_args* args, hymeta_stream_t stream);
 
 /* Mixture of experts whose choice is a table lookup by token id: table [vocab, top_k] names each

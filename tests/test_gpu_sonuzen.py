@@ -152,7 +152,8 @@ def _paged_attention(q, k, v, dtype, block_size, portions, scale, r1, r2, qw, kw
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 16, 24), (3, 3, 8, 8), (6, 1, 40, 16), (2, 1, 128, 128)])
+@pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 16, 24), (3, 3, 8, 8), (6, 1, 40, 16), (2, 1, 128, 128), (4, 2, 64, 64), (8, 2, 64, 128),
+                                     (5, 1, 128, 64)])
 def test_sink_attention_over_pages_in_portions(dtype, H, G, D, Dv):
     g = torch.Generator().manual_seed(H * 31 + D)
     T, eps, scale = 75, 1e-5, 0.3
@@ -175,11 +176,12 @@ def test_sink_attention_over_pages_in_portions(dtype, H, G, D, Dv):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_a_key_far_back_decides_the_output(dtype):
+@pytest.mark.parametrize("D", [16, 64])
+def test_a_key_far_back_decides_the_output(dtype, D):
     """Hundreds of keys, one of which (far back, on a page border) matches the last queries many times better than the
     rest even after the distance bias: the output is that key's value row, in a prompt's portion and for a decoded token."""
     g = torch.Generator().manual_seed(5)
-    T, H, G, D, Dv, bs = 700, 2, 1, 16, 16, 64
+    T, H, G, Dv, bs = 700, 2, 1, D, 64
     q, k, v = bf16_values(T, H, D, std=0.3, gen=g), bf16_values(T, G, D, std=0.3, gen=g), bf16_values(T, G, Dv, gen=g)
     far = 64                                                    # first row of the second page
     k[far] = 0
@@ -261,6 +263,8 @@ MODELS = {
                                            logit_scale=1.0),
     "one_tap_one_head": dict(layers=("attention",), heads=1, kv_heads=1, dim=32, vdim=16, taps=1, loop=(0, 1, 2), experts=2, top=2,
                              ff=40, width=72, scale=0.4),
+    "matrix_core_head_sizes": dict(layers=("attention", "mingru", "attention"), loop=(1, 3, 2), width=128, heads=4, kv_heads=2, dim=64,
+                                   vdim=128, ff=64, experts=4, top=2),
     "no_convolution": dict(layers=("mingru", "attention"), taps=0, width=128, ff=64, heads=8, kv_heads=2, dim=16, vdim=32),
 }
 

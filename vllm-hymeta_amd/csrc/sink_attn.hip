@@ -128,6 +128,342 @@ __global__ __launch_bounds__(64) void sink_attention_rows_kernel(hymeta_sink_att
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// bf16 on the matrix cores.  A wave owns 32 "rows" (two blocks of 16): in a prompt's portion 32 consecutive query
+// rows of one head, in a decode step the query heads of one key/value head (they share every key and value row they
+// read).  Keys come in tiles of 64 through LDS: the key rows as they lie in the pages, the value rows transposed, so
+// that both are read as MFMA operands with 8- and 16-byte LDS loads.
+//
+//   S^T[key][row] = K[key][:] . Q[row][:]           v_mfma_f32_16x16x32_bf16, A = K fragment, B = Q fragment
+//   O^T[c][row]  += V^T[c][key] P^T[key][row]       A = V^T fragment, B = P^T
+//
+// The transposed forms make the result layout of the first product (a lane holds 4 consecutive keys of one row) the
+// B-operand layout of the second, so the weights never leave their registers, and they leave the row statistics in the
+// lane that owns the row in both products.  The weights stay fp32-exact through the bf16 matrix product: p = hi + lo
+// with hi = bf16(p), lo = bf16(p - hi), two products (relative error of p 2^-17 instead of 2^-9).
+// ------------------------------------------------------------------------------------------------
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4v mfma16(bf16x8 a, bf16x8 b, f32x4v c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+constexpr int kTileKeys = 64;
+constexpr int kRowsPerWave = 32;
+
+template <int D, int DV>
+struct MfmaSmem {
+  static constexpr int kPitchK = D + 8;               // bf16 elements per key row (16-byte reads of 16 rows: no bank conflict)
+  static constexpr int kPitchV = kTileKeys + 8;       // bf16 elements per value channel
+  uint16_t k[kTileKeys * kPitchK];
+  uint16_t vt[DV * kPitchV];
+};
+
+// Stage keys [j0, j0 + 64) of a sequence's key/value head g: 16-byte chunks, consecutive threads on consecutive chunks
+// of a row (a key row and its value row are one contiguous run in a page).  Keys past `last` are zero.
+template <int D, int DV, int Threads>
+__device__ __forceinline__ void stage_tile(MfmaSmem<D, DV>& sm, const hymeta_sink_attention_args& a, const int32_t* bt, int g,
+                                           int j0, int last) {
+  constexpr int kChunksPerRow = (D + DV) / 8;
+  constexpr int kChunks = kTileKeys * kChunksPerRow;
+  const uint16_t* cache = static_cast<const uint16_t*>(a.kv_cache);
+  const int64_t row_elems = static_cast<int64_t>(a.num_kv_heads) * (D + DV);
+#pragma unroll 4
+  for (int idx = threadIdx.x; idx < kChunks; idx += Threads) {
+    const int r = idx / kChunksPerRow, ch = idx % kChunksPerRow;
+    const int j = j0 + r;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (j <= last) {
+      const int64_t blk = bt[j / a.block_size];
+      v = ld16g(cache + (blk * a.block_size + j % a.block_size) * row_elems + static_cast<int64_t>(g) * (D + DV) + ch * 8);
+    }
+    if (ch < D / 8) {
+      st16(&sm.k[r * MfmaSmem<D, DV>::kPitchK + ch * 8], v);
+    } else {
+      const int c0 = (ch - D / 8) * 8;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        sm.vt[(c0 + 2 * e) * MfmaSmem<D, DV>::kPitchV + r] = static_cast<uint16_t>(v[e] & 0xffffu);
+        sm.vt[(c0 + 2 * e + 1) * MfmaSmem<D, DV>::kPitchV + r] = static_cast<uint16_t>(v[e] >> 16);
+      }
+    }
+  }
+}
+
+// The rows of one wave against the staged tile.  Per row block rb and lane: row = 16 rb + lane % 16.
+template <int D, int DV>
+struct WaveRows {
+  bf16x8 q[2][D / 32];
+  f32x4v o[2][DV / 16];
+  float m[2], l[2];            // running maximum of the row; this lane's share of the denominator
+  int pos[2];                  // position of the row's query (-1: no such row)
+  float ba[2], bb[2];
+};
+
+template <int D, int DV>
+__device__ __forceinline__ void attend_tile(WaveRows<D, DV>& w, const MfmaSmem<D, DV>& sm, const hymeta_sink_attention_args& a,
+                                            int j0) {
+  const int lane = threadIdx.x & 63, n = lane & 15, g4 = lane >> 4;
+  constexpr int PK = MfmaSmem<D, DV>::kPitchK, PV = MfmaSmem<D, DV>::kPitchV;
+  f32x4v s[2][4];
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) s[rb][ks] = f32x4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+    for (int st = 0; st < D / 32; ++st) {
+      const bf16x8 kf = __builtin_bit_cast(bf16x8, ld16(&sm.k[(16 * ks + n) * PK + 32 * st + 8 * g4]));
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) s[rb][ks] = mfma16(kf, w.q[rb][st], s[rb][ks]);
+    }
+  // lane holds, per row block, the scores of its row (n) against keys j0 + 16 ks + 4 g4 + r
+  bf16x8 phi[2][2], plo[2][2];
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb) {
+    const int pos = w.pos[rb];
+    const int first = a.window_left >= 0 ? pos - a.window_left : 0;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int j = j0 + 16 * ks + 4 * g4 + r;
+        float sc = s[rb][ks][r] * a.scale;
+        if (a.bias_mode == HYMETA_BIAS_LOG_DISTANCE) sc -= w.ba[rb] * __logf(1.f + w.bb[rb] * static_cast<float>(pos - j));
+        sc = (j <= pos && j >= first) ? sc : -INFINITY;
+        s[rb][ks][r] = sc;
+        mx = fmaxf(mx, sc);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(w.m[rb], mx);
+    // a row with nothing visible so far and no sink keeps m = -inf: every weight and the correction are then 0
+    const float corr = m_new == -INFINITY ? 0.f : __expf(w.m[rb] - m_new);
+    float sum = 0.f;
+    uint16_t hi[16], lo[16];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float p = m_new == -INFINITY ? 0.f : __expf(s[rb][ks][r] - m_new);
+        sum += p;
+        const uint16_t h16 = f2bf(p);
+        hi[4 * ks + r] = h16;
+        lo[4 * ks + r] = f2bf(p - bf2f(h16));
+      }
+    w.l[rb] = w.l[rb] * corr + sum;
+    w.m[rb] = m_new;
+#pragma unroll
+    for (int cb = 0; cb < DV / 16; ++cb) w.o[rb][cb] *= corr;
+#pragma unroll
+    for (int kp = 0; kp < 2; ++kp) {
+      bf16x8 ph, pl;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        ph[e] = static_cast<short>(hi[8 * kp + e]);     // keys 16 (2 kp) + 4 g4 + e, then 16 (2 kp + 1) + 4 g4 + e - 4
+        pl[e] = static_cast<short>(lo[8 * kp + e]);
+      }
+      phi[rb][kp] = ph;
+      plo[rb][kp] = pl;
+    }
+  }
+#pragma unroll
+  for (int cb = 0; cb < DV / 16; ++cb)
+#pragma unroll
+    for (int kp = 0; kp < 2; ++kp) {
+      const uint16_t* vrow = &sm.vt[(16 * cb + n) * PV + 32 * kp + 4 * g4];
+      const u32x2 v0 = *reinterpret_cast<const u32x2*>(vrow), v1 = *reinterpret_cast<const u32x2*>(vrow + 16);
+      const u32x4 vv = {v0[0], v0[1], v1[0], v1[1]};
+      const bf16x8 vf = __builtin_bit_cast(bf16x8, vv);
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
+        w.o[rb][cb] = mfma16(vf, phi[rb][kp], w.o[rb][cb]);
+        w.o[rb][cb] = mfma16(vf, plo[rb][kp], w.o[rb][cb]);
+      }
+    }
+}
+
+template <int D, int DV>
+__device__ __forceinline__ void load_q(WaveRows<D, DV>& w, int rb, const uint16_t* qrow) {
+  const int g4 = (threadIdx.x & 63) >> 4;
+#pragma unroll
+  for (int st = 0; st < D / 32; ++st)
+    w.q[rb][st] = qrow ? __builtin_bit_cast(bf16x8, ld16g(qrow + 32 * st + 8 * g4)) : bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+}
+
+// Portions of prompts: grid = (tiles of 128 rows, heads, sequences); sequences with one row are left to the decode form.
+template <int D, int DV>
+__global__ __launch_bounds__(256) void sink_attention_prefill_mfma_kernel(hymeta_sink_attention_args a) {
+  __shared__ MfmaSmem<D, DV> sm;
+  const int s = blockIdx.z, h = blockIdx.y;
+  const int row0 = a.query_start_loc[s];
+  const int q = a.query_start_loc[s + 1] - row0;
+  if (q <= 1 || static_cast<int>(blockIdx.x) * 128 >= q) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g4 = lane >> 4;
+  const int g = h / (a.num_heads / a.num_kv_heads);
+  const int ctx = a.seq_lens[s] - q;
+  const int32_t* bt = a.block_tables + static_cast<int64_t>(s) * a.block_table_stride;
+  WaveRows<D, DV> w;
+  const int wrow = blockIdx.x * 128 + wave * kRowsPerWave;
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb) {
+    const int r = wrow + 16 * rb + n;
+    const bool ok = r < q;
+    w.pos[rb] = ok ? ctx + r : -1;
+    w.ba[rb] = a.bias_mode ? a.bias_a[h] : 0.f;
+    w.bb[rb] = a.bias_mode ? a.bias_b[h] : 0.f;
+    w.m[rb] = a.sink ? 0.f : -INFINITY;
+    w.l[rb] = (a.sink && g4 == 0) ? 1.f : 0.f;        // the sink's exp(0 - 0), counted once per row
+    load_q<D, DV>(w, rb, ok ? static_cast<const uint16_t*>(a.q) + static_cast<int64_t>(row0 + r) * a.q_stride_t + static_cast<int64_t>(h) * D : nullptr);
+#pragma unroll
+    for (int cb = 0; cb < DV / 16; ++cb) w.o[rb][cb] = f32x4v{0.f, 0.f, 0.f, 0.f};
+  }
+  const int block_last = ctx + min(q, static_cast<int>(blockIdx.x) * 128 + 128) - 1;      // last key any row of the block sees
+  const int wave_last = ctx + min(q, wrow + kRowsPerWave) - 1;
+  int j_first = 0;
+  if (a.window_left >= 0) j_first = max(0, ctx + static_cast<int>(blockIdx.x) * 128 - a.window_left) / kTileKeys * kTileKeys;
+  for (int j0 = j_first; j0 <= block_last; j0 += kTileKeys) {
+    __syncthreads();
+    stage_tile<D, DV, 256>(sm, a, bt, g, j0, block_last);
+    __syncthreads();
+    if (wrow < q && j0 <= wave_last) attend_tile<D, DV>(w, sm, a, j0);
+  }
+  if (wrow >= q) return;
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb) {
+    float l = w.l[rb];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const int r = wrow + 16 * rb + n;
+    if (r >= q) continue;
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    uint16_t* out = static_cast<uint16_t*>(a.out) + (static_cast<int64_t>(row0 + r) * a.num_heads + h) * DV;
+#pragma unroll
+    for (int cb = 0; cb < DV / 16; ++cb) {
+      const f32x4v o = w.o[rb][cb] * inv;
+      *reinterpret_cast<u32x2*>(out + 16 * cb + 4 * g4) = u32x2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
+    }
+  }
+}
+
+// Decode: one wave per (sequence with one row, key/value head, slice of the keys); rows = the group's query heads.  Writes
+// the slice's (maximum, denominator, weighted values) per head; the combine kernel merges the slices and the sink.
+// Partial of a (sequence, key/value head, slice): per query head of the group DV weighted values, then the slice's
+// maximum and denominator, rows padded to whole 16 bytes.
+__host__ __device__ inline size_t partial_row_floats(int dv) { return static_cast<size_t>(dv) + 4; }
+
+template <int D, int DV>
+__global__ __launch_bounds__(64) void sink_attention_decode_mfma_kernel(hymeta_sink_attention_args a, int splits, int tiles_per_split) {
+  __shared__ MfmaSmem<D, DV> sm;
+  const int s = blockIdx.z, g = blockIdx.y, split = blockIdx.x;
+  const int t = a.query_start_loc[s];
+  if (a.query_start_loc[s + 1] - t != 1) return;
+  const int pos = a.seq_lens[s] - 1;
+  const int HG = a.num_heads / a.num_kv_heads;
+  const int lane = threadIdx.x & 63, n = lane & 15, g4 = lane >> 4;
+  int j_lo = split * tiles_per_split * kTileKeys, j_hi = min(pos, j_lo + tiles_per_split * kTileKeys - 1);
+  int first = 0;
+  if (a.window_left >= 0) first = max(0, pos - a.window_left);
+  float* part = static_cast<float*>(a.workspace) +
+                ((static_cast<size_t>(s) * a.num_kv_heads + g) * splits + split) * (HG * partial_row_floats(DV));
+  const int32_t* bt = a.block_tables + static_cast<int64_t>(s) * a.block_table_stride;
+  WaveRows<D, DV> w;
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb) {
+    const int r = 16 * rb + n;
+    const bool ok = r < HG;
+    const int h = g * HG + (ok ? r : 0);
+    w.pos[rb] = ok ? pos : -1;
+    w.ba[rb] = a.bias_mode ? a.bias_a[h] : 0.f;
+    w.bb[rb] = a.bias_mode ? a.bias_b[h] : 0.f;
+    w.m[rb] = -INFINITY;
+    w.l[rb] = 0.f;
+    load_q<D, DV>(w, rb, ok ? static_cast<const uint16_t*>(a.q) + static_cast<int64_t>(t) * a.q_stride_t + static_cast<int64_t>(h) * D : nullptr);
+#pragma unroll
+    for (int cb = 0; cb < DV / 16; ++cb) w.o[rb][cb] = f32x4v{0.f, 0.f, 0.f, 0.f};
+  }
+  for (int j0 = j_lo; j0 <= j_hi; j0 += kTileKeys) {
+    if (j0 + kTileKeys - 1 < first) continue;
+    __syncthreads();
+    stage_tile<D, DV, 64>(sm, a, bt, g, j0, j_hi);
+    __syncthreads();
+    attend_tile<D, DV>(w, sm, a, j0);
+  }
+#pragma unroll
+  for (int rb = 0; rb < 2; ++rb) {
+    float l = w.l[rb];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const int r = 16 * rb + n;
+    if (r >= HG) continue;
+    float* pr = part + r * partial_row_floats(DV);
+    if (g4 == 0) pr[DV] = w.m[rb], pr[DV + 1] = l;
+#pragma unroll
+    for (int cb = 0; cb < DV / 16; ++cb)
+      *reinterpret_cast<f32x4v*>(pr + 16 * cb + 4 * g4) = w.o[rb][cb];
+  }
+}
+
+// grid = (sequences, heads), 64 threads: merge the slices of a decode row, add the sink, normalise, store bf16.
+__global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymeta_sink_attention_args a, int splits) {
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int t = a.query_start_loc[s];
+  if (a.query_start_loc[s + 1] - t != 1) return;
+  const int HG = a.num_heads / a.num_kv_heads, g = h / HG, r = h % HG, DV = a.v_dim;
+  const size_t stride = HG * partial_row_floats(DV);
+  const float* base = static_cast<const float*>(a.workspace) + (static_cast<size_t>(s) * a.num_kv_heads + g) * splits * stride +
+                      r * partial_row_floats(DV);
+  float m = a.sink ? 0.f : -INFINITY;
+  for (int sp = 0; sp < splits; ++sp) m = fmaxf(m, base[sp * stride + DV]);
+  float l = a.sink ? __expf(0.f - m) : 0.f;
+  for (int sp = 0; sp < splits; ++sp) {
+    const float ms = base[sp * stride + DV];
+    if (ms != -INFINITY) l += base[sp * stride + DV + 1] * __expf(ms - m);
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  uint16_t* out = static_cast<uint16_t*>(a.out) + (static_cast<int64_t>(t) * a.num_heads + h) * DV;
+  for (int c = threadIdx.x; c < DV; c += 64) {
+    float acc = 0.f;
+    for (int sp = 0; sp < splits; ++sp) {
+      const float ms = base[sp * stride + DV];
+      if (ms != -INFINITY) acc += base[sp * stride + c] * __expf(ms - m);
+    }
+    out[c] = f2bf(acc * inv);
+  }
+}
+
+inline bool mfma_shape(const hymeta_sink_attention_args& a) {
+  const bool dims = (a.head_dim == 64 || a.head_dim == 128) && (a.v_dim == 64 || a.v_dim == 128);
+  return a.act_dtype == HYMETA_BF16 && dims && a.num_heads / a.num_kv_heads <= kRowsPerWave && a.q_stride_t % 8 == 0 &&
+         (reinterpret_cast<uintptr_t>(a.q) | reinterpret_cast<uintptr_t>(a.kv_cache) | reinterpret_cast<uintptr_t>(a.out)) % 16 == 0;
+}
+
+inline int decode_splits(int num_seqs, int num_kv_heads, int max_seq_len) {
+  const int tiles = (max_seq_len + kTileKeys - 1) / kTileKeys;
+  int splits = (2048 + num_seqs * num_kv_heads - 1) / (num_seqs * num_kv_heads);     // about eight waves per compute unit
+  splits = splits < 1 ? 1 : splits;
+  return splits > tiles ? (tiles < 1 ? 1 : tiles) : splits;
+}
+
+template <int D, int DV>
+int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st) {
+  if (a.max_query_len > 1) {
+    const dim3 grid((a.max_query_len + 127) / 128, a.num_heads, a.num_seqs);
+    hipLaunchKernelGGL((sink_attention_prefill_mfma_kernel<D, DV>), grid, dim3(256), 0, st, a);
+  }
+  // sequences with a single row: every step but a pure prompt step has some; a prompt of one token is one too
+  const int splits = decode_splits(a.num_seqs, a.num_kv_heads, a.max_seq_len);
+  const int tiles = (a.max_seq_len + kTileKeys - 1) / kTileKeys;
+  const int tiles_per_split = (tiles + splits - 1) / splits;
+  hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV>), dim3(splits, a.num_kv_heads, a.num_seqs), dim3(64), 0, st, a, splits,
+                     tiles_per_split);
+  hipLaunchKernelGGL(sink_attention_decode_combine_kernel, dim3(a.num_seqs, a.num_heads), dim3(64), 0, st, a, splits);
+  return launch_status();
+}
+
 }  // namespace
 
 }  // namespace hymeta
@@ -151,9 +487,11 @@ extern "C" int hymeta_qk_norm_cache(const hymeta_qk_norm_cache_args* args, hymet
   return launch_status();
 }
 
-extern "C" size_t hymeta_sink_attention_workspace_bytes(int32_t num_tokens, int32_t num_heads, int32_t v_dim, int32_t max_seq_len) {
-  (void)num_tokens, (void)num_heads, (void)v_dim, (void)max_seq_len;
-  return 0;
+extern "C" size_t hymeta_sink_attention_workspace_bytes(int32_t num_seqs, int32_t num_heads, int32_t num_kv_heads, int32_t v_dim,
+                                                        int32_t max_seq_len) {
+  if (num_seqs <= 0 || num_heads <= 0 || num_kv_heads <= 0 || v_dim <= 0) return 0;
+  const int splits = decode_splits(num_seqs, num_kv_heads, max_seq_len < 1 ? 1 : max_seq_len);
+  return static_cast<size_t>(num_seqs) * splits * num_heads * partial_row_floats(v_dim) * sizeof(float);
 }
 
 extern "C" int hymeta_sink_attention(const hymeta_sink_attention_args* args, hymeta_stream_t stream) {
@@ -171,6 +509,15 @@ extern "C" int hymeta_sink_attention(const hymeta_sink_attention_args* args, hym
   if (a.bias_mode != HYMETA_BIAS_NONE && (!a.bias_a || !a.bias_b)) return HYMETA_ERR_INVALID_ARG;
   if (a.num_heads > 65535) return HYMETA_ERR_UNSUPPORTED;
   hipStream_t st = begin_launches(stream);
+  if (mfma_shape(a) && a.max_query_len >= 1 && a.max_seq_len >= 1) {
+    const size_t need = hymeta_sink_attention_workspace_bytes(a.num_seqs, a.num_heads, a.num_kv_heads, a.v_dim, a.max_seq_len);
+    if (!a.workspace || a.workspace_bytes < need) return HYMETA_ERR_WORKSPACE;
+    if (a.num_seqs > 65535 || a.num_heads > 65535) return HYMETA_ERR_UNSUPPORTED;
+    if (a.head_dim == 64 && a.v_dim == 64) return launch_mfma<64, 64>(a, st);
+    if (a.head_dim == 64 && a.v_dim == 128) return launch_mfma<64, 128>(a, st);
+    if (a.head_dim == 128 && a.v_dim == 64) return launch_mfma<128, 64>(a, st);
+    return launch_mfma<128, 128>(a, st);
+  }
   const dim3 grid(a.num_tokens, a.num_heads);
   if (a.act_dtype == HYMETA_BF16) hipLaunchKernelGGL(sink_attention_rows_kernel<ActBf16>, grid, dim3(64), 0, st, a);
   else hipLaunchKernelGGL(sink_attention_rows_kernel<ActF32>, grid, dim3(64), 0, st, a);

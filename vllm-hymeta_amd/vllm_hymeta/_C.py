@@ -455,7 +455,7 @@ _SIGNATURES = {
     "hymeta_norm_residual": (C.c_int, [C.POINTER(NormResidualArgs), _ptr]),
     "hymeta_mingru": (C.c_int, [C.POINTER(MinGruArgs), _ptr]),
     "hymeta_qk_norm_cache": (C.c_int, [C.POINTER(QkNormCacheArgs), _ptr]),
-    "hymeta_sink_attention_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32]),
+    "hymeta_sink_attention_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32, _i32]),
     "hymeta_sink_attention": (C.c_int, [C.POINTER(SinkAttentionArgs), _ptr]),
     "hymeta_moe_route_table": (C.c_int, [C.POINTER(MoeRouteTableArgs), _ptr]),
     "hymeta_moe_gemm_any": (C.c_int, [C.POINTER(MoeGemmAnyArgs), _ptr]),

@@ -1616,7 +1616,7 @@ def sink_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_tables: torch.
     a = _C.SinkAttentionArgs()
     a.q, a.kv_cache, a.out, a.block_tables = _p(q), _p(kv_cache), _p(out), _p(block_tables)
     a.query_start_loc, a.seq_lens, a.bias_a, a.bias_b = _p(query_start_loc), _p(seq_lens), _p(bias_a), _p(bias_b)
-    nbytes = int(lib.hymeta_sink_attention_workspace_bytes(T, H, v_dim, max_seq_len))
+    nbytes = int(lib.hymeta_sink_attention_workspace_bytes(S, H, num_kv_heads, v_dim, max_seq_len))
     if nbytes:
         ws = _workspace(q.device, nbytes, "sink_attention")
         a.workspace, a.workspace_bytes = _p(ws), ws.numel()
