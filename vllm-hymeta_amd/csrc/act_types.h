@@ -12,6 +12,8 @@ struct ActBf16 {
   static __device__ __forceinline__ float ld(const elem* p) { return bf2f(*p); }
   static __device__ __forceinline__ void st(elem* p, float v) { *p = f2bf(v); }
   static __device__ __forceinline__ float round(float v) { return bf16_round(v); }
+  // fp32 in, fp32 out, the hardware's exponential (about 2 ulp): where the inputs carry 8 bits
+  static __device__ __forceinline__ float sigmoid(float x) { return 1.f / (1.f + __expf(-x)); }
 };
 
 struct ActF32 {
@@ -20,6 +22,7 @@ struct ActF32 {
   static __device__ __forceinline__ float ld(const elem* p) { return *p; }
   static __device__ __forceinline__ void st(elem* p, float v) { *p = v; }
   static __device__ __forceinline__ float round(float v) { return v; }
+  static __device__ __forceinline__ float sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
 };
 
 inline bool act_dtype_ok(int d) { return d == HYMETA_BF16 || d == HYMETA_F32; }

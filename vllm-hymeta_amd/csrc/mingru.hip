@@ -32,21 +32,34 @@ __global__ __launch_bounds__(64 * Waves) void mingru_kernel(hymeta_mingru_args a
   const elem* zug = static_cast<const elem*>(a.zug);
   elem* out = static_cast<elem*>(a.out);
 
+  // the raw projections of a round are loaded one round ahead of their use
+  float rz[kRun], ru[kRun], rg[kRun];
+  auto load = [&](int base, float (&z)[kRun], float (&u)[kRun], float (&g)[kRun]) {
+    const int lo = base + wave * kRun;
+#pragma unroll
+    for (int l = 0; l < kRun; ++l) {
+      z[l] = u[l] = g[l] = 0.f;
+      if (live && lo + l < q) {
+        const elem* r = zug + (row0 + lo + l) * a.zug_stride_t;
+        z[l] = A::ld(r + c), u[l] = A::ld(r + W + c), g[l] = A::ld(r + 2 * W + c);
+      }
+    }
+  };
+  load(0, rz, ru, rg);
   for (int base = 0; base < q; base += kRun * Waves) {
     const int lo = base + wave * kRun;
+    float nz[kRun], nu[kRun], ng[kRun];
+    if (base + kRun * Waves < q) load(base + kRun * Waves, nz, nu, ng);
     float av[kRun], bv[kRun], gv[kRun];
 #pragma unroll
     for (int l = 0; l < kRun; ++l) {
       av[l] = 1.f, bv[l] = 0.f, gv[l] = 0.f;
       if (live && lo + l < q) {
-        const elem* r = zug + (row0 + lo + l) * a.zug_stride_t;
-        const float z = sigmoid_exact(A::ld(r + c));
-        const float u = A::ld(r + W + c);
-        const float cand = u >= 0.f ? u + 0.5f : sigmoid_exact(u);
-        const float g = A::ld(r + 2 * W + c);
+        const float z = A::sigmoid(rz[l]);
+        const float cand = ru[l] >= 0.f ? ru[l] + 0.5f : A::sigmoid(ru[l]);
         av[l] = 1.f - z;
         bv[l] = z * cand;
-        gv[l] = g * sigmoid_exact(g);
+        gv[l] = rg[l] * A::sigmoid(rg[l]);
       }
     }
     float S = carry;
@@ -75,6 +88,8 @@ __global__ __launch_bounds__(64 * Waves) void mingru_kernel(hymeta_mingru_args a
       if (live && lo + l < q) A::st(out + (row0 + lo + l) * W + c, S * gv[l]);
     }
     if (Waves == 1) carry = S;
+#pragma unroll
+    for (int l = 0; l < kRun; ++l) rz[l] = nz[l], ru[l] = nu[l], rg[l] = ng[l];
   }
   if (live && slot >= 0 && wave == 0) a.state[static_cast<int64_t>(slot) * W + c] = carry;
 }

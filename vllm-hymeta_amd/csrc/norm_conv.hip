@@ -25,32 +25,26 @@ __global__ __launch_bounds__(kNormThreads) void embed_rows_kernel(hymeta_embed_r
   for (int c = threadIdx.x; c < a.width; c += kNormThreads) out[c] = A::ld(row + c) + (a.add ? a.add[c] : 0.f);
 }
 
-// 1 / sqrt(mean(row^2) + eps) of an fp32 row, the same value in every thread.
-__device__ __forceinline__ float inv_rms(const float* row, int width, float eps, float* red) {
-  float ss = 0.f;
-  for (int c = threadIdx.x; c < width; c += kNormThreads) {
-    const float v = row[c];
-    ss += v * v;
-  }
-  ss = block_sum<kNormWaves>(ss, red);
-  return 1.f / sqrtf(ss / static_cast<float>(width) + eps);
-}
+constexpr int kMaxRows = 2 * (HYMETA_CONV_MAX_TAPS - 1);      // rows whose statistic one workgroup may need
 
 // One workgroup per token row.  Rows 1 .. taps - 2 of a portion are computed by the workgroup of its row 0, which is
 // also the only one that touches the sequence's convolution state: it reads the old rows for the portion's first
 // outputs and then writes the new ones.  A thread owns its channels in all of this, so no other thread waits for its
-// reads or sees its writes.
+// reads or sees its writes.  The sums of squares of all the rows a workgroup needs (its own and its predecessors',
+// for the first workgroup also the rows that become the new state) are reduced together, one barrier pair.
 template <typename A>
 __global__ __launch_bounds__(kNormThreads) void norm_conv_kernel(hymeta_norm_conv_args a) {
   typedef typename A::elem elem;
-  __shared__ float red[kNormWaves];
+  __shared__ float red[kNormWaves][kMaxRows];
   const int t = blockIdx.x;
   const int taps = a.conv_weight ? a.taps : 1;
   const int hist = taps - 1;
   int s = 0, i = 0, q = 1, ctx = 0, slot = -1;
   int64_t row0 = t;
   if (hist > 0) {
-    s = seq_of_row(a.query_start_loc, a.num_seqs, t);
+    // a step of single rows (decode) has sequence t at row t: two independent loads instead of a search
+    if (t < a.num_seqs && a.query_start_loc[t] == t && a.query_start_loc[t + 1] == t + 1) s = t;
+    else s = seq_of_row(a.query_start_loc, a.num_seqs, t);
     row0 = a.query_start_loc[s];
     i = t - static_cast<int>(row0);
     q = a.query_start_loc[s + 1] - static_cast<int>(row0);
@@ -61,54 +55,73 @@ __global__ __launch_bounds__(kNormThreads) void norm_conv_kernel(hymeta_norm_con
   elem* state = (hist > 0 && a.conv_state && slot >= 0)
                     ? static_cast<elem*>(a.conv_state) + static_cast<int64_t>(slot) * hist * a.width : nullptr;
   const bool carried = state != nullptr && ctx > 0;
-  const int todo = (hist > 0 && i == 0) ? min(hist, q) : 1;
+  const bool first = hist > 0 && i == 0;
+  const int todo = first ? min(hist, q) : 1;
 
-  for (int ii = i; ii < i + todo; ++ii) {
-    // the normed rows ii - hist .. ii of the portion (those at or after its start)
-    float inv[HYMETA_CONV_MAX_TAPS];
-    for (int j = 0; j < taps; ++j) {
-      const int k = ii - hist + j;
-      inv[j] = 0.f;
-      if (k >= 0) inv[j] = inv_rms(a.x + (row0 + k) * a.x_stride_t, a.width, a.eps, red);
-    }
-    elem* out = static_cast<elem*>(a.out) + (row0 + ii) * static_cast<int64_t>(a.width);
-    for (int c = threadIdx.x; c < a.width; c += kNormThreads) {
-      const float w = a.weight_offset + a.weight[c];
-      const float n = A::round(a.x[(row0 + ii) * a.x_stride_t + c] * inv[hist] * w);
-      float acc = n;
-      if (a.conv_weight != nullptr) {
-        const float* cw = a.conv_weight + static_cast<int64_t>(c) * taps;
-        acc = fmaf(cw[hist], n, acc);
-        for (int j = 0; j < hist; ++j) {
-          const int k = ii - hist + j;
-          float v = 0.f;
-          if (k >= 0) v = A::round(a.x[(row0 + k) * a.x_stride_t + c] * inv[j] * w);
-          else if (carried) v = A::ld(state + static_cast<int64_t>(hist + k) * a.width + c);
-          acc = fmaf(cw[j], v, acc);
-        }
+  // portion rows whose statistic is needed: [lo1, lo1 + n1) for the outputs, [lo2, lo2 + n2) more for the new state
+  const int lo1 = first ? 0 : i - hist, n1 = first ? todo : taps;
+  const int lo2 = max(todo, q - hist), n2 = (first && state != nullptr) ? max(0, q - lo2) : 0;
+  float ss[kMaxRows];
+#pragma unroll
+  for (int r = 0; r < kMaxRows; ++r) ss[r] = 0.f;
+  for (int c = threadIdx.x; c < a.width; c += kNormThreads) {
+#pragma unroll
+    for (int r = 0; r < kMaxRows; ++r) {
+      if (r < n1 + n2) {
+        const int k = r < n1 ? lo1 + r : lo2 + (r - n1);
+        const float v = a.x[(row0 + k) * a.x_stride_t + c];
+        ss[r] = fmaf(v, v, ss[r]);
       }
-      A::st(out + c, acc);
     }
   }
-
-  if (hist > 0 && i == 0 && state != nullptr) {
-    // new state row r = the normed row at portion index q - hist + r; indices before the portion come from the old
-    // state (row q + r, which lies after the row being written: ascending r never reads a row already replaced)
-    float inv[HYMETA_CONV_MAX_TAPS];
-    for (int r = 0; r < hist; ++r) {
-      const int k = q - hist + r;
-      inv[r] = 0.f;
-      if (k >= 0) inv[r] = inv_rms(a.x + (row0 + k) * a.x_stride_t, a.width, a.eps, red);
+#pragma unroll
+  for (int r = 0; r < kMaxRows; ++r)
+    if (r < n1 + n2) {
+      const float v = wave_sum(ss[r]);
+      if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6][r] = v;
     }
-    for (int c = threadIdx.x; c < a.width; c += kNormThreads) {
-      const float w = a.weight_offset + a.weight[c];
-      for (int r = 0; r < hist; ++r) {
-        const int k = q - hist + r;
-        float v = 0.f;
-        if (k >= 0) v = A::round(a.x[(row0 + k) * a.x_stride_t + c] * inv[r] * w);
-        else if (carried) v = A::ld(state + static_cast<int64_t>(hist + k) * a.width + c);
-        A::st(state + static_cast<int64_t>(r) * a.width + c, v);
+  __syncthreads();
+  float inv[kMaxRows];
+#pragma unroll
+  for (int r = 0; r < kMaxRows; ++r) {
+    inv[r] = 0.f;
+    if (r < n1 + n2) {
+      float v = 0.f;
+#pragma unroll
+      for (int w = 0; w < kNormWaves; ++w) v += red[w][r];
+      inv[r] = 1.f / sqrtf(v / static_cast<float>(a.width) + a.eps);
+    }
+  }
+  // the statistic of portion row k (k in one of the two ranges)
+  auto inv_of = [&](int k) -> float {
+    const int r = (k >= lo1 && k < lo1 + n1) ? k - lo1 : n1 + (k - lo2);
+    float v = 0.f;
+#pragma unroll
+    for (int u = 0; u < kMaxRows; ++u) v = (u == r) ? inv[u] : v;
+    return v;
+  };
+
+  for (int c = threadIdx.x; c < a.width; c += kNormThreads) {
+    const float w = a.weight_offset + a.weight[c];
+    const float* cw = a.conv_weight ? a.conv_weight + static_cast<int64_t>(c) * taps : nullptr;
+    // the normed value of portion row k of this channel (k < 0: from the carried state, or zero)
+    auto normed = [&](int k) -> float {
+      if (k >= 0) return A::round(a.x[(row0 + k) * a.x_stride_t + c] * inv_of(k) * w);
+      return carried ? A::ld(state + static_cast<int64_t>(hist + k) * a.width + c) : 0.f;
+    };
+    for (int ii = i; ii < i + todo; ++ii) {
+      const float n = normed(ii);
+      float acc = n;
+      if (cw != nullptr) {
+        acc = fmaf(cw[hist], n, acc);
+        for (int j = 0; j < hist; ++j) acc = fmaf(cw[j], normed(ii - hist + j), acc);
       }
+      A::st(static_cast<elem*>(a.out) + (row0 + ii) * static_cast<int64_t>(a.width) + c, acc);
+    }
+    if (first && state != nullptr) {
+      // new state row r = the normed row at portion index q - hist + r; indices before the portion come from the old
+      // state (row q + r, which lies after the row being written: ascending r never reads a row already replaced)
+      for (int r = 0; r < hist; ++r) A::st(state + static_cast<int64_t>(r) * a.width + c, normed(q - hist + r));
     }
   }
 }

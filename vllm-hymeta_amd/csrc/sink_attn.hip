@@ -160,77 +160,125 @@ struct MfmaSmem {
   uint16_t vt[DV * kPitchV];
 };
 
-// Stage keys [j0, j0 + 64) of a sequence's key/value head g: 16-byte chunks, consecutive threads on consecutive chunks
-// of a row (a key row and its value row are one contiguous run in a page).  Keys past `last` are zero.
+// Staging of keys [j0, j0 + 64) of a sequence's key/value head g, in two halves so that the loads of the next tile
+// are in flight while the current one is multiplied: `issue` reads 16-byte chunks into registers (keys past `last` read
+// as zero), `commit` stores them into LDS.  A key row goes in as it is.  The value rows go in transposed: a thread takes
+// the same 8 channels of 4 consecutive keys (4 chunks), which are 8 runs of 4 keys in the transposed image, one 8-byte
+// store each.  The 4-key groups of a channel are permuted by the channel's chunk number (XOR), which spreads the stores
+// of threads that hold the same keys over the banks; the reader applies the same permutation.
 template <int D, int DV, int Threads>
-__device__ __forceinline__ void stage_tile(MfmaSmem<D, DV>& sm, const hymeta_sink_attention_args& a, const int32_t* bt, int g,
-                                           int j0, int last) {
-  constexpr int kChunksPerRow = (D + DV) / 8;
-  constexpr int kChunks = kTileKeys * kChunksPerRow;
-  const uint16_t* cache = static_cast<const uint16_t*>(a.kv_cache);
-  const int64_t row_elems = static_cast<int64_t>(a.num_kv_heads) * (D + DV);
-#pragma unroll 4
-  for (int idx = threadIdx.x; idx < kChunks; idx += Threads) {
-    const int r = idx / kChunksPerRow, ch = idx % kChunksPerRow;
-    const int j = j0 + r;
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (j <= last) {
-      const int64_t blk = bt[j / a.block_size];
-      v = ld16g(cache + (blk * a.block_size + j % a.block_size) * row_elems + static_cast<int64_t>(g) * (D + DV) + ch * 8);
-    }
-    if (ch < D / 8) {
-      st16(&sm.k[r * MfmaSmem<D, DV>::kPitchK + ch * 8], v);
-    } else {
-      const int c0 = (ch - D / 8) * 8;
+struct TileStage {
+  static constexpr int kKeyChunksPerRow = D / 8, kValChunksPerRow = DV / 8;
+  static constexpr int kKeyPerThread = kTileKeys * kKeyChunksPerRow / Threads;
+  static constexpr int kValBlocks = (kTileKeys / 4) * kValChunksPerRow;       // (4 keys) x (8 channels) each
+  static_assert(kTileKeys * kKeyChunksPerRow % Threads == 0 && kValBlocks <= Threads, "the staging roles fit the workgroup");
+  u32x4 rk[kKeyPerThread];
+  u32x4 rv[4];
+
+  static __device__ __forceinline__ const uint16_t* row_ptr(const hymeta_sink_attention_args& a, const int32_t* bt, int g, int j) {
+    // pages hold a power of two of rows here (the host sends other sizes to the plain kernel): shift and mask
+    const int page_shift = __builtin_ctz(a.block_size), page_mask = a.block_size - 1;
+    const int64_t blk = bt[j >> page_shift];
+    return static_cast<const uint16_t*>(a.kv_cache) +
+           ((blk << page_shift) + (j & page_mask)) * (static_cast<int64_t>(a.num_kv_heads) * (D + DV)) + static_cast<int64_t>(g) * (D + DV);
+  }
+
+  __device__ __forceinline__ void issue(const hymeta_sink_attention_args& a, const int32_t* bt, int g, int j0, int last) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        sm.vt[(c0 + 2 * e) * MfmaSmem<D, DV>::kPitchV + r] = static_cast<uint16_t>(v[e] & 0xffffu);
-        sm.vt[(c0 + 2 * e + 1) * MfmaSmem<D, DV>::kPitchV + r] = static_cast<uint16_t>(v[e] >> 16);
+    for (int i = 0; i < kKeyPerThread; ++i) {
+      const int idx = i * Threads + threadIdx.x;
+      const int j = j0 + idx / kKeyChunksPerRow;
+      rk[i] = u32x4{0u, 0u, 0u, 0u};
+      if (j <= last) rk[i] = ld16g(row_ptr(a, bt, g, j) + (idx % kKeyChunksPerRow) * 8);
+    }
+    if (static_cast<int>(threadIdx.x) < kValBlocks) {
+      const int ch = threadIdx.x % kValChunksPerRow, grp = threadIdx.x / kValChunksPerRow;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = j0 + 4 * grp + i;
+        rv[i] = u32x4{0u, 0u, 0u, 0u};
+        if (j <= last) rv[i] = ld16g(row_ptr(a, bt, g, j) + D + ch * 8);
       }
     }
   }
-}
 
-// The rows of one wave against the staged tile.  Per row block rb and lane: row = 16 rb + lane % 16.
-template <int D, int DV>
-struct WaveRows {
-  bf16x8 q[2][D / 32];
-  f32x4v o[2][DV / 16];
-  float m[2], l[2];            // running maximum of the row; this lane's share of the denominator
-  int pos[2];                  // position of the row's query (-1: no such row)
-  float ba[2], bb[2];
+  __device__ __forceinline__ void commit(MfmaSmem<D, DV>& sm) const {
+#pragma unroll
+    for (int i = 0; i < kKeyPerThread; ++i) {
+      const int idx = i * Threads + threadIdx.x;
+      st16(&sm.k[(idx / kKeyChunksPerRow) * MfmaSmem<D, DV>::kPitchK + (idx % kKeyChunksPerRow) * 8], rk[i]);
+    }
+    if (static_cast<int>(threadIdx.x) < kValBlocks) {
+      const int ch = threadIdx.x % kValChunksPerRow, grp = threadIdx.x / kValChunksPerRow;
+      uint16_t* dst = &sm.vt[(8 * ch) * MfmaSmem<D, DV>::kPitchV + 4 * (grp ^ (ch & 15))];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int dw = e >> 1;
+        u32x2 v;
+        if (e & 1) {
+          v[0] = (rv[0][dw] >> 16) | (rv[1][dw] & 0xffff0000u);
+          v[1] = (rv[2][dw] >> 16) | (rv[3][dw] & 0xffff0000u);
+        } else {
+          v[0] = (rv[0][dw] & 0xffffu) | (rv[1][dw] << 16);
+          v[1] = (rv[2][dw] & 0xffffu) | (rv[3][dw] << 16);
+        }
+        *reinterpret_cast<u32x2*>(dst + e * MfmaSmem<D, DV>::kPitchV) = v;
+      }
+    }
+  }
 };
 
+// Where the 4-key group `grp` (0 .. 15) of value channel c lies in the transposed image.
 template <int D, int DV>
-__device__ __forceinline__ void attend_tile(WaveRows<D, DV>& w, const MfmaSmem<D, DV>& sm, const hymeta_sink_attention_args& a,
-                                            int j0) {
+__device__ __forceinline__ const uint16_t* vt_group(const MfmaSmem<D, DV>& sm, int c, int grp) {
+  return &sm.vt[c * MfmaSmem<D, DV>::kPitchV + 4 * (grp ^ ((c >> 3) & 15))];
+}
+
+// The rows of one wave against the staged tile.  RB row blocks of 16 (row = 16 rb + lane % 16); the wave takes NKS of the
+// tile's four 16-key subtiles, from ks_lo on (a prompt's wave all four, a decode wave one: the four waves of a decode
+// workgroup split every tile between them and each keeps statistics of its own).
+template <int D, int DV, int RB>
+struct WaveRows {
+  bf16x8 q[RB][D / 32];
+  f32x4v o[RB][DV / 16];
+  float m[RB], l[RB];          // running maximum of the row; this lane's share of the denominator
+  int pos[RB];                 // position of the row's query (-1: no such row)
+  float ba[RB], bb[RB];
+};
+
+typedef short bf16x4 __attribute__((ext_vector_type(4)));
+
+template <int D, int DV, int RB, int NKS>
+__device__ __forceinline__ void attend_tile(WaveRows<D, DV, RB>& w, const MfmaSmem<D, DV>& sm, const hymeta_sink_attention_args& a,
+                                            int j0, int ks_lo) {
+  static_assert(NKS == 4 || NKS == 1, "all of a tile's subtiles or one");
   const int lane = threadIdx.x & 63, n = lane & 15, g4 = lane >> 4;
-  constexpr int PK = MfmaSmem<D, DV>::kPitchK, PV = MfmaSmem<D, DV>::kPitchV;
-  f32x4v s[2][4];
+  constexpr int PK = MfmaSmem<D, DV>::kPitchK;
+  f32x4v s[RB][NKS];
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb)
+  for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) s[rb][ks] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    for (int ks = 0; ks < NKS; ++ks) s[rb][ks] = f32x4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks)
+  for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
     for (int st = 0; st < D / 32; ++st) {
-      const bf16x8 kf = __builtin_bit_cast(bf16x8, ld16(&sm.k[(16 * ks + n) * PK + 32 * st + 8 * g4]));
+      const bf16x8 kf = __builtin_bit_cast(bf16x8, ld16(&sm.k[(16 * (ks_lo + ks) + n) * PK + 32 * st + 8 * g4]));
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb) s[rb][ks] = mfma16(kf, w.q[rb][st], s[rb][ks]);
+      for (int rb = 0; rb < RB; ++rb) s[rb][ks] = mfma16(kf, w.q[rb][st], s[rb][ks]);
     }
-  // lane holds, per row block, the scores of its row (n) against keys j0 + 16 ks + 4 g4 + r
-  bf16x8 phi[2][2], plo[2][2];
+  // lane holds, per row block, the scores of its row (n) against keys j0 + 16 (ks_lo + ks) + 4 g4 + r
+  uint32_t phi[RB][NKS][2], plo[RB][NKS][2];       // the weights' bf16 high and low parts, two per dword
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
+  for (int rb = 0; rb < RB; ++rb) {
     const int pos = w.pos[rb];
     const int first = a.window_left >= 0 ? pos - a.window_left : 0;
     float mx = -INFINITY;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
+    for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int j = j0 + 16 * ks + 4 * g4 + r;
+        const int j = j0 + 16 * (ks_lo + ks) + 4 * g4 + r;
         float sc = s[rb][ks][r] * a.scale;
         if (a.bias_mode == HYMETA_BIAS_LOG_DISTANCE) sc -= w.ba[rb] * __logf(1.f + w.bb[rb] * static_cast<float>(pos - j));
         sc = (j <= pos && j >= first) ? sc : -INFINITY;
@@ -243,136 +291,145 @@ __device__ __forceinline__ void attend_tile(WaveRows<D, DV>& w, const MfmaSmem<D
     // a row with nothing visible so far and no sink keeps m = -inf: every weight and the correction are then 0
     const float corr = m_new == -INFINITY ? 0.f : __expf(w.m[rb] - m_new);
     float sum = 0.f;
-    uint16_t hi[16], lo[16];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
+    for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float p = m_new == -INFINITY ? 0.f : __expf(s[rb][ks][r] - m_new);
-        sum += p;
-        const uint16_t h16 = f2bf(p);
-        hi[4 * ks + r] = h16;
-        lo[4 * ks + r] = f2bf(p - bf2f(h16));
+      for (int r2 = 0; r2 < 2; ++r2) {
+        float p[2], res[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          p[u] = m_new == -INFINITY ? 0.f : __expf(s[rb][ks][2 * r2 + u] - m_new);
+          sum += p[u];
+          res[u] = p[u] - bf16_round(p[u]);
+        }
+        phi[rb][ks][r2] = pack_bf16x2(p[0], p[1]);
+        plo[rb][ks][r2] = pack_bf16x2(res[0], res[1]);
       }
     w.l[rb] = w.l[rb] * corr + sum;
     w.m[rb] = m_new;
 #pragma unroll
     for (int cb = 0; cb < DV / 16; ++cb) w.o[rb][cb] *= corr;
+  }
+  if constexpr (NKS == 4) {
 #pragma unroll
-    for (int kp = 0; kp < 2; ++kp) {
-      bf16x8 ph, pl;
+    for (int cb = 0; cb < DV / 16; ++cb)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        ph[e] = static_cast<short>(hi[8 * kp + e]);     // keys 16 (2 kp) + 4 g4 + e, then 16 (2 kp + 1) + 4 g4 + e - 4
-        pl[e] = static_cast<short>(lo[8 * kp + e]);
+      for (int kp = 0; kp < 2; ++kp) {
+        // k index 8 g4 + e of the product: keys 16 (2 kp) + 4 g4 + e for e < 4, 16 (2 kp + 1) + 4 g4 + e - 4 after
+        const u32x2 v0 = *reinterpret_cast<const u32x2*>(vt_group<D, DV>(sm, 16 * cb + n, 8 * kp + g4));
+        const u32x2 v1 = *reinterpret_cast<const u32x2*>(vt_group<D, DV>(sm, 16 * cb + n, 8 * kp + 4 + g4));
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, (u32x4{v0[0], v0[1], v1[0], v1[1]}));
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          const bf16x8 ph = __builtin_bit_cast(bf16x8, (u32x4{phi[rb][2 * kp][0], phi[rb][2 * kp][1], phi[rb][2 * kp + 1][0], phi[rb][2 * kp + 1][1]}));
+          const bf16x8 pl = __builtin_bit_cast(bf16x8, (u32x4{plo[rb][2 * kp][0], plo[rb][2 * kp][1], plo[rb][2 * kp + 1][0], plo[rb][2 * kp + 1][1]}));
+          w.o[rb][cb] = mfma16(vf, ph, w.o[rb][cb]);
+          w.o[rb][cb] = mfma16(vf, pl, w.o[rb][cb]);
+        }
       }
-      phi[rb][kp] = ph;
-      plo[rb][kp] = pl;
+  } else {
+#pragma unroll
+    for (int cb = 0; cb < DV / 16; ++cb) {
+      const bf16x4 vf = __builtin_bit_cast(bf16x4, *reinterpret_cast<const u32x2*>(vt_group<D, DV>(sm, 16 * cb + n, 4 * ks_lo + g4)));
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const bf16x4 ph = __builtin_bit_cast(bf16x4, (u32x2{phi[rb][0][0], phi[rb][0][1]}));
+        const bf16x4 pl = __builtin_bit_cast(bf16x4, (u32x2{plo[rb][0][0], plo[rb][0][1]}));
+        w.o[rb][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, ph, w.o[rb][cb], 0, 0, 0);
+        w.o[rb][cb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pl, w.o[rb][cb], 0, 0, 0);
+      }
     }
   }
-#pragma unroll
-  for (int cb = 0; cb < DV / 16; ++cb)
-#pragma unroll
-    for (int kp = 0; kp < 2; ++kp) {
-      const uint16_t* vrow = &sm.vt[(16 * cb + n) * PV + 32 * kp + 4 * g4];
-      const u32x2 v0 = *reinterpret_cast<const u32x2*>(vrow), v1 = *reinterpret_cast<const u32x2*>(vrow + 16);
-      const u32x4 vv = {v0[0], v0[1], v1[0], v1[1]};
-      const bf16x8 vf = __builtin_bit_cast(bf16x8, vv);
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb) {
-        w.o[rb][cb] = mfma16(vf, phi[rb][kp], w.o[rb][cb]);
-        w.o[rb][cb] = mfma16(vf, plo[rb][kp], w.o[rb][cb]);
-      }
-    }
 }
 
-template <int D, int DV>
-__device__ __forceinline__ void load_q(WaveRows<D, DV>& w, int rb, const uint16_t* qrow) {
+template <int D, int DV, int RB>
+__device__ __forceinline__ void load_q(WaveRows<D, DV, RB>& w, int rb, const uint16_t* qrow) {
   const int g4 = (threadIdx.x & 63) >> 4;
 #pragma unroll
   for (int st = 0; st < D / 32; ++st)
     w.q[rb][st] = qrow ? __builtin_bit_cast(bf16x8, ld16g(qrow + 32 * st + 8 * g4)) : bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
 }
 
+constexpr int kPrefillWaves = 8;                        // 16 rows each
+constexpr int kPrefillRows = 16 * kPrefillWaves;
+
 // Portions of prompts: grid = (tiles of 128 rows, heads, sequences); sequences with one row are left to the decode form.
 template <int D, int DV>
-__global__ __launch_bounds__(256) void sink_attention_prefill_mfma_kernel(hymeta_sink_attention_args a) {
+__global__ __launch_bounds__(64 * kPrefillWaves) void sink_attention_prefill_mfma_kernel(hymeta_sink_attention_args a) {
   __shared__ MfmaSmem<D, DV> sm;
   const int s = blockIdx.z, h = blockIdx.y;
   const int row0 = a.query_start_loc[s];
   const int q = a.query_start_loc[s + 1] - row0;
-  if (q <= 1 || static_cast<int>(blockIdx.x) * 128 >= q) return;
+  if (q <= 1 || static_cast<int>(blockIdx.x) * kPrefillRows >= q) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g4 = lane >> 4;
   const int g = h / (a.num_heads / a.num_kv_heads);
   const int ctx = a.seq_lens[s] - q;
   const int32_t* bt = a.block_tables + static_cast<int64_t>(s) * a.block_table_stride;
-  WaveRows<D, DV> w;
-  const int wrow = blockIdx.x * 128 + wave * kRowsPerWave;
+  WaveRows<D, DV, 1> w;
+  const int wrow = blockIdx.x * kPrefillRows + wave * 16;
+  const int r = wrow + n;
+  const bool ok = r < q;
+  w.pos[0] = ok ? ctx + r : -1;
+  w.ba[0] = a.bias_mode ? a.bias_a[h] : 0.f;
+  w.bb[0] = a.bias_mode ? a.bias_b[h] : 0.f;
+  w.m[0] = a.sink ? 0.f : -INFINITY;
+  w.l[0] = (a.sink && g4 == 0) ? 1.f : 0.f;        // the sink's exp(0 - 0), counted once per row
+  load_q<D, DV, 1>(w, 0, ok ? static_cast<const uint16_t*>(a.q) + static_cast<int64_t>(row0 + r) * a.q_stride_t + static_cast<int64_t>(h) * D : nullptr);
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
-    const int r = wrow + 16 * rb + n;
-    const bool ok = r < q;
-    w.pos[rb] = ok ? ctx + r : -1;
-    w.ba[rb] = a.bias_mode ? a.bias_a[h] : 0.f;
-    w.bb[rb] = a.bias_mode ? a.bias_b[h] : 0.f;
-    w.m[rb] = a.sink ? 0.f : -INFINITY;
-    w.l[rb] = (a.sink && g4 == 0) ? 1.f : 0.f;        // the sink's exp(0 - 0), counted once per row
-    load_q<D, DV>(w, rb, ok ? static_cast<const uint16_t*>(a.q) + static_cast<int64_t>(row0 + r) * a.q_stride_t + static_cast<int64_t>(h) * D : nullptr);
-#pragma unroll
-    for (int cb = 0; cb < DV / 16; ++cb) w.o[rb][cb] = f32x4v{0.f, 0.f, 0.f, 0.f};
-  }
-  const int block_last = ctx + min(q, static_cast<int>(blockIdx.x) * 128 + 128) - 1;      // last key any row of the block sees
-  const int wave_last = ctx + min(q, wrow + kRowsPerWave) - 1;
+  for (int cb = 0; cb < DV / 16; ++cb) w.o[0][cb] = f32x4v{0.f, 0.f, 0.f, 0.f};
+  const int block_last = ctx + min(q, static_cast<int>(blockIdx.x) * kPrefillRows + kPrefillRows) - 1;      // last key any row of the block sees
+  const int wave_last = ctx + min(q, wrow + 16) - 1;
   int j_first = 0;
-  if (a.window_left >= 0) j_first = max(0, ctx + static_cast<int>(blockIdx.x) * 128 - a.window_left) / kTileKeys * kTileKeys;
+  if (a.window_left >= 0) j_first = max(0, ctx + static_cast<int>(blockIdx.x) * kPrefillRows - a.window_left) / kTileKeys * kTileKeys;
+  TileStage<D, DV, 64 * kPrefillWaves> stage;
+  stage.issue(a, bt, g, j_first, block_last);
   for (int j0 = j_first; j0 <= block_last; j0 += kTileKeys) {
+    __syncthreads();                   // every wave is done with the tile before
+    stage.commit(sm);
     __syncthreads();
-    stage_tile<D, DV, 256>(sm, a, bt, g, j0, block_last);
-    __syncthreads();
-    if (wrow < q && j0 <= wave_last) attend_tile<D, DV>(w, sm, a, j0);
+    if (j0 + kTileKeys <= block_last) stage.issue(a, bt, g, j0 + kTileKeys, block_last);
+    if (wrow < q && j0 <= wave_last) attend_tile<D, DV, 1, 4>(w, sm, a, j0, 0);
   }
-  if (wrow >= q) return;
+  if (!ok) return;
+  float l = w.l[0];
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  uint16_t* out = static_cast<uint16_t*>(a.out) + (static_cast<int64_t>(row0 + r) * a.num_heads + h) * DV;
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
-    float l = w.l[rb];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
-    const int r = wrow + 16 * rb + n;
-    if (r >= q) continue;
-    const float inv = l > 0.f ? 1.f / l : 0.f;
-    uint16_t* out = static_cast<uint16_t*>(a.out) + (static_cast<int64_t>(row0 + r) * a.num_heads + h) * DV;
-#pragma unroll
-    for (int cb = 0; cb < DV / 16; ++cb) {
-      const f32x4v o = w.o[rb][cb] * inv;
-      *reinterpret_cast<u32x2*>(out + 16 * cb + 4 * g4) = u32x2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
-    }
+  for (int cb = 0; cb < DV / 16; ++cb) {
+    const f32x4v o = w.o[0][cb] * inv;
+    *reinterpret_cast<u32x2*>(out + 16 * cb + 4 * g4) = u32x2{pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3])};
   }
 }
 
-// Decode: one wave per (sequence with one row, key/value head, slice of the keys); rows = the group's query heads.  Writes
-// the slice's (maximum, denominator, weighted values) per head; the combine kernel merges the slices and the sink.
-// Partial of a (sequence, key/value head, slice): per query head of the group DV weighted values, then the slice's
+// Partial of a (sequence, key/value head, slice, wave): per query head of the group DV weighted values, then the
 // maximum and denominator, rows padded to whole 16 bytes.
 __host__ __device__ inline size_t partial_row_floats(int dv) { return static_cast<size_t>(dv) + 4; }
+constexpr int kDecodeWaves = 4;
 
-template <int D, int DV>
-__global__ __launch_bounds__(64) void sink_attention_decode_mfma_kernel(hymeta_sink_attention_args a, int splits, int tiles_per_split) {
+// Decode: a workgroup per (sequence with one row, key/value head, slice of the keys); rows = the group's query heads; the
+// four waves share the staged tiles and take a 16-key subtile each.  Every wave writes its (maximum, denominator,
+// weighted values) per head; the combine kernel merges them and the sink.
+template <int D, int DV, int RB>
+__global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_kernel(hymeta_sink_attention_args a, int splits, int tiles_per_split) {
   __shared__ MfmaSmem<D, DV> sm;
   const int s = blockIdx.z, g = blockIdx.y, split = blockIdx.x;
   const int t = a.query_start_loc[s];
   if (a.query_start_loc[s + 1] - t != 1) return;
   const int pos = a.seq_lens[s] - 1;
   const int HG = a.num_heads / a.num_kv_heads;
-  const int lane = threadIdx.x & 63, n = lane & 15, g4 = lane >> 4;
-  int j_lo = split * tiles_per_split * kTileKeys, j_hi = min(pos, j_lo + tiles_per_split * kTileKeys - 1);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g4 = lane >> 4;
+  int j_lo = split * tiles_per_split * kTileKeys;
+  const int j_hi = min(pos, j_lo + tiles_per_split * kTileKeys - 1);
   int first = 0;
   if (a.window_left >= 0) first = max(0, pos - a.window_left);
   float* part = static_cast<float*>(a.workspace) +
-                ((static_cast<size_t>(s) * a.num_kv_heads + g) * splits + split) * (HG * partial_row_floats(DV));
+                (((static_cast<size_t>(s) * a.num_kv_heads + g) * splits + split) * kDecodeWaves + wave) * (HG * partial_row_floats(DV));
   const int32_t* bt = a.block_tables + static_cast<int64_t>(s) * a.block_table_stride;
-  WaveRows<D, DV> w;
+  WaveRows<D, DV, RB> w;
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
+  for (int rb = 0; rb < RB; ++rb) {
     const int r = 16 * rb + n;
     const bool ok = r < HG;
     const int h = g * HG + (ok ? r : 0);
@@ -381,19 +438,22 @@ __global__ __launch_bounds__(64) void sink_attention_decode_mfma_kernel(hymeta_s
     w.bb[rb] = a.bias_mode ? a.bias_b[h] : 0.f;
     w.m[rb] = -INFINITY;
     w.l[rb] = 0.f;
-    load_q<D, DV>(w, rb, ok ? static_cast<const uint16_t*>(a.q) + static_cast<int64_t>(t) * a.q_stride_t + static_cast<int64_t>(h) * D : nullptr);
+    load_q<D, DV, RB>(w, rb, ok ? static_cast<const uint16_t*>(a.q) + static_cast<int64_t>(t) * a.q_stride_t + static_cast<int64_t>(h) * D : nullptr);
 #pragma unroll
     for (int cb = 0; cb < DV / 16; ++cb) w.o[rb][cb] = f32x4v{0.f, 0.f, 0.f, 0.f};
   }
+  if (j_lo < first) j_lo = first / kTileKeys * kTileKeys;      // tiles wholly before the window are not read
+  TileStage<D, DV, 64 * kDecodeWaves> stage;
+  if (j_lo <= j_hi) stage.issue(a, bt, g, j_lo, j_hi);
   for (int j0 = j_lo; j0 <= j_hi; j0 += kTileKeys) {
-    if (j0 + kTileKeys - 1 < first) continue;
     __syncthreads();
-    stage_tile<D, DV, 64>(sm, a, bt, g, j0, j_hi);
+    stage.commit(sm);
     __syncthreads();
-    attend_tile<D, DV>(w, sm, a, j0);
+    if (j0 + kTileKeys <= j_hi) stage.issue(a, bt, g, j0 + kTileKeys, j_hi);
+    if (j0 + 16 * wave <= j_hi) attend_tile<D, DV, RB, 1>(w, sm, a, j0, wave);
   }
 #pragma unroll
-  for (int rb = 0; rb < 2; ++rb) {
+  for (int rb = 0; rb < RB; ++rb) {
     float l = w.l[rb];
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
@@ -409,6 +469,7 @@ __global__ __launch_bounds__(64) void sink_attention_decode_mfma_kernel(hymeta_s
 
 // grid = (sequences, heads), 64 threads: merge the slices of a decode row, add the sink, normalise, store bf16.
 __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymeta_sink_attention_args a, int splits) {
+  splits *= kDecodeWaves;                // every wave of a slice wrote a partial of its own
   const int s = blockIdx.x, h = blockIdx.y;
   const int t = a.query_start_loc[s];
   if (a.query_start_loc[s + 1] - t != 1) return;
@@ -438,12 +499,13 @@ __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymet
 inline bool mfma_shape(const hymeta_sink_attention_args& a) {
   const bool dims = (a.head_dim == 64 || a.head_dim == 128) && (a.v_dim == 64 || a.v_dim == 128);
   return a.act_dtype == HYMETA_BF16 && dims && a.num_heads / a.num_kv_heads <= kRowsPerWave && a.q_stride_t % 8 == 0 &&
+         (a.block_size & (a.block_size - 1)) == 0 &&
          (reinterpret_cast<uintptr_t>(a.q) | reinterpret_cast<uintptr_t>(a.kv_cache) | reinterpret_cast<uintptr_t>(a.out)) % 16 == 0;
 }
 
 inline int decode_splits(int num_seqs, int num_kv_heads, int max_seq_len) {
   const int tiles = (max_seq_len + kTileKeys - 1) / kTileKeys;
-  int splits = (2048 + num_seqs * num_kv_heads - 1) / (num_seqs * num_kv_heads);     // about eight waves per compute unit
+  int splits = (1024 + num_seqs * num_kv_heads - 1) / (num_seqs * num_kv_heads);     // about four workgroups per compute unit
   splits = splits < 1 ? 1 : splits;
   return splits > tiles ? (tiles < 1 ? 1 : tiles) : splits;
 }
@@ -451,15 +513,18 @@ inline int decode_splits(int num_seqs, int num_kv_heads, int max_seq_len) {
 template <int D, int DV>
 int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st) {
   if (a.max_query_len > 1) {
-    const dim3 grid((a.max_query_len + 127) / 128, a.num_heads, a.num_seqs);
-    hipLaunchKernelGGL((sink_attention_prefill_mfma_kernel<D, DV>), grid, dim3(256), 0, st, a);
+    const dim3 grid((a.max_query_len + kPrefillRows - 1) / kPrefillRows, a.num_heads, a.num_seqs);
+    hipLaunchKernelGGL((sink_attention_prefill_mfma_kernel<D, DV>), grid, dim3(64 * kPrefillWaves), 0, st, a);
   }
   // sequences with a single row: every step but a pure prompt step has some; a prompt of one token is one too
   const int splits = decode_splits(a.num_seqs, a.num_kv_heads, a.max_seq_len);
   const int tiles = (a.max_seq_len + kTileKeys - 1) / kTileKeys;
   const int tiles_per_split = (tiles + splits - 1) / splits;
-  hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV>), dim3(splits, a.num_kv_heads, a.num_seqs), dim3(64), 0, st, a, splits,
-                     tiles_per_split);
+  const dim3 grid(splits, a.num_kv_heads, a.num_seqs);
+  if (a.num_heads / a.num_kv_heads <= 16)
+    hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 1>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split);
+  else
+    hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 2>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split);
   hipLaunchKernelGGL(sink_attention_decode_combine_kernel, dim3(a.num_seqs, a.num_heads), dim3(64), 0, st, a, splits);
   return launch_status();
 }
@@ -491,7 +556,7 @@ extern "C" size_t hymeta_sink_attention_workspace_bytes(int32_t num_seqs, int32_
                                                         int32_t max_seq_len) {
   if (num_seqs <= 0 || num_heads <= 0 || num_kv_heads <= 0 || v_dim <= 0) return 0;
   const int splits = decode_splits(num_seqs, num_kv_heads, max_seq_len < 1 ? 1 : max_seq_len);
-  return static_cast<size_t>(num_seqs) * splits * num_heads * partial_row_floats(v_dim) * sizeof(float);
+  return static_cast<size_t>(num_seqs) * splits * kDecodeWaves * num_heads * partial_row_floats(v_dim) * sizeof(float);
 }
 
 extern "C" int hymeta_sink_attention(const hymeta_sink_attention_args* args, hymeta_stream_t stream) {
