@@ -67,6 +67,33 @@ def test_norm_conv_in_portions_carries_its_state(dtype, taps, width):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("taps,width", [(3, 96), (4, 272), (2, 64), (5, 40), (3, 4200)])
+def test_norm_conv_of_long_steps(dtype, taps, width):
+    """Steps of a thousand rows and more run in strips of rows whose inputs are read once; strips that hold a portion's
+    first rows or a boundary between two sequences do not.  Two sequences in one step, then their next portions."""
+    from vllm_hymeta import hip_ops
+    g = torch.Generator().manual_seed(taps + width)
+    lens = [1301, 702]
+    xs = [torch.randn(n, width, generator=g, dtype=torch.float64) for n in lens]
+    w, cw, eps = torch.randn(width, generator=g).double() * 0.2, torch.randn(width, taps, generator=g).double() * 0.5, 1e-5
+    refs = [causal_conv_add_ref(norm_one_plus_ref(x, w, eps), cw) for x in xs]
+    state = torch.zeros(2, taps - 1, width, dtype=dtype, device=DEV)
+    first = [1027, 601]                                   # the second sequence starts inside a strip
+    step1 = torch.cat([xs[0][:first[0]], xs[1][:first[1]]]).float().to(DEV)
+    args = (w.float().to(DEV), eps, dtype, 1.0, cw.float().to(DEV).contiguous(), state)
+    out1 = hip_ops.norm_conv(step1, *args, i32([0, first[0], first[0] + first[1]]), i32([0, 0]), i32([1, 0]))
+    step2 = torch.cat([xs[1][first[1]:], xs[0][first[0]:], ]).float().to(DEV)
+    n1, n0 = lens[1] - first[1], lens[0] - first[0]
+    out2 = hip_ops.norm_conv(step2, *args, i32([0, n1, n1 + n0]), i32([first[1], first[0]]), i32([0, 1]))
+    assert rel_err(torch.cat([out1[:first[0]], out2[n1:]]), refs[0]) < TOL[dtype]
+    assert rel_err(torch.cat([out1[first[0]:], out2[:n1]]), refs[1]) < TOL[dtype]
+    # the strip form and the row form give the same values: the same rows in a step too short for strips
+    short = hip_ops.norm_conv(step1[100:900].contiguous(), *args[:5], None, i32([0, 800]), i32([0]), None)
+    long_ = hip_ops.norm_conv(step1[100:1300].contiguous(), *args[:5], None, i32([0, 1200]), i32([0]), None)
+    assert rel_err(long_[8:800], short[8:800]) < (1e-6 if dtype == torch.float32 else 4e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_plain_norm_and_output_norm_with_residual(dtype):
     from vllm_hymeta import hip_ops
     g = torch.Generator().manual_seed(3)
@@ -156,7 +183,7 @@ def _paged_attention(q, k, v, dtype, block_size, portions, scale, r1, r2, qw, kw
                                      (5, 1, 128, 64)])
 def test_sink_attention_over_pages_in_portions(dtype, H, G, D, Dv):
     g = torch.Generator().manual_seed(H * 31 + D)
-    T, eps, scale = 75, 1e-5, 0.3
+    T, eps, scale = 150, 1e-5, 0.3
     q, k, v = bf16_values(T, H, D, gen=g), bf16_values(T, G, D, gen=g), bf16_values(T, G, Dv, gen=g)
     qw, kw = 1 + bf16_values(D, std=0.2, gen=g), 1 + bf16_values(D, std=0.2, gen=g)
     r1, r2 = torch.rand(H, generator=g).double() + 0.2, torch.rand(H, generator=g).double() * 0.5 + 0.05
@@ -164,9 +191,10 @@ def test_sink_attention_over_pages_in_portions(dtype, H, G, D, Dv):
     if dtype == torch.bfloat16:      # what the cache and the query rows hold
         qn, kn = qn.to(dtype).double(), kn.to(dtype).double()
     ref = sink_attention_ref(qn, kn, v, scale, r1, r2)
-    for portions in ([T], [40] + [1] * 35, [2, 14, 16, 1, 31, 2, 9]):       # page size 16: portions end on, before and after borders
-        out = _paged_attention(q, k, v, dtype, 16, portions, scale, r1, r2, qw, kw, eps, shuffle_seed=len(portions))
-        assert rel_err(out, ref) < (3e-5 if dtype == torch.float32 else 1e-2), portions
+    for portions in ([T], [115] + [1] * 35, [2, 14, 16, 1, 31, 2, 9, 64, 11]):       # page size 16: portions end on, before and after borders
+        for page in (16, 64):
+            out = _paged_attention(q, k, v, dtype, page, portions, scale, r1, r2, qw, kw, eps, shuffle_seed=len(portions))
+            assert rel_err(out, ref) < (3e-5 if dtype == torch.float32 else 1e-2), (portions, page)
     no_sink = sink_attention_ref(qn, kn, v, scale, r1, r2, sink=False)
     assert rel_err(ref, no_sink) > 0.05           # the inputs do tell a softmax with a sink from one without
     out = _paged_attention(q, k, v, dtype, 16, [T], scale, r1, r2, qw, kw, eps, sink=False)
@@ -298,8 +326,10 @@ def test_model_schedules_agree_with_the_whole_prompt(name, dtype):
     refs = {k: sonuzen_ref(cfg, weights, t) for k, t in seqs.items()}
     tol_ref = 3e-5 if dtype == torch.float32 else 4e-2
     tol_self = 3e-5 if dtype == torch.float32 else 3e-2
-    # page size 16, pool of 12 pages = 192 tokens: never room for everything at once
-    eng = build_engine(cfg, weights, dtype, max_tokens=192, block_size=16, max_num_seqs=4)
+    # pool of 12 pages of 16 tokens (64 for the model whose attention runs on the matrix cores, where a page holds a whole
+    # tile of keys): never room for everything at once
+    page = 64 if name == "matrix_core_head_sizes" else 16
+    eng = build_engine(cfg, weights, dtype, max_tokens=12 * page, block_size=page, max_num_seqs=4)
     whole = {}
     for k, t in seqs.items():
         whole[k] = eng.run_batch([(f"w{k}", t, list(range(len(t))))])

@@ -25,7 +25,10 @@ __global__ __launch_bounds__(kNormThreads) void embed_rows_kernel(hymeta_embed_r
   for (int c = threadIdx.x; c < a.width; c += kNormThreads) out[c] = A::ld(row + c) + (a.add ? a.add[c] : 0.f);
 }
 
-constexpr int kMaxRows = 2 * (HYMETA_CONV_MAX_TAPS - 1);      // rows whose statistic one workgroup may need
+__device__ __forceinline__ int seq_of_row_fast(const hymeta_norm_conv_args& a, int t);
+
+constexpr int kMaxRows = 2 * (HYMETA_CONV_MAX_TAPS - 1);
+constexpr int kRowUnroll = 16;               // channels per thread whose loads are issued together (width <= 4096)      // rows whose statistic one workgroup may need
 
 // One workgroup per token row.  Rows 1 .. taps - 2 of a portion are computed by the workgroup of its row 0, which is
 // also the only one that touches the sequence's convolution state: it reads the old rows for the portion's first
@@ -33,18 +36,15 @@ constexpr int kMaxRows = 2 * (HYMETA_CONV_MAX_TAPS - 1);      // rows whose stat
 // reads or sees its writes.  The sums of squares of all the rows a workgroup needs (its own and its predecessors',
 // for the first workgroup also the rows that become the new state) are reduced together, one barrier pair.
 template <typename A>
-__global__ __launch_bounds__(kNormThreads) void norm_conv_kernel(hymeta_norm_conv_args a) {
+__device__ __forceinline__ void norm_conv_row(const hymeta_norm_conv_args& a, int t, float (*red)[kMaxRows]) {
   typedef typename A::elem elem;
-  __shared__ float red[kNormWaves][kMaxRows];
-  const int t = blockIdx.x;
   const int taps = a.conv_weight ? a.taps : 1;
   const int hist = taps - 1;
   int s = 0, i = 0, q = 1, ctx = 0, slot = -1;
   int64_t row0 = t;
   if (hist > 0) {
     // a step of single rows (decode) has sequence t at row t: two independent loads instead of a search
-    if (t < a.num_seqs && a.query_start_loc[t] == t && a.query_start_loc[t + 1] == t + 1) s = t;
-    else s = seq_of_row(a.query_start_loc, a.num_seqs, t);
+    s = seq_of_row_fast(a, t);
     row0 = a.query_start_loc[s];
     i = t - static_cast<int>(row0);
     q = a.query_start_loc[s + 1] - static_cast<int>(row0);
@@ -64,7 +64,8 @@ __global__ __launch_bounds__(kNormThreads) void norm_conv_kernel(hymeta_norm_con
   float ss[kMaxRows];
 #pragma unroll
   for (int r = 0; r < kMaxRows; ++r) ss[r] = 0.f;
-  for (int c = threadIdx.x; c < a.width; c += kNormThreads) {
+  // (the first 16 channels of a thread with every load in flight at once; wider rows go on in a plain loop)
+  auto stats_at = [&](int c) {
 #pragma unroll
     for (int r = 0; r < kMaxRows; ++r) {
       if (r < n1 + n2) {
@@ -73,7 +74,13 @@ __global__ __launch_bounds__(kNormThreads) void norm_conv_kernel(hymeta_norm_con
         ss[r] = fmaf(v, v, ss[r]);
       }
     }
+  };
+#pragma unroll
+  for (int u = 0; u < kRowUnroll; ++u) {
+    const int c = threadIdx.x + u * kNormThreads;
+    if (c < a.width) stats_at(c);
   }
+  for (int c = threadIdx.x + kRowUnroll * kNormThreads; c < a.width; c += kNormThreads) stats_at(c);
 #pragma unroll
   for (int r = 0; r < kMaxRows; ++r)
     if (r < n1 + n2) {
@@ -101,7 +108,7 @@ __global__ __launch_bounds__(kNormThreads) void norm_conv_kernel(hymeta_norm_con
     return v;
   };
 
-  for (int c = threadIdx.x; c < a.width; c += kNormThreads) {
+  auto emit_at = [&](int c) {
     const float w = a.weight_offset + a.weight[c];
     const float* cw = a.conv_weight ? a.conv_weight + static_cast<int64_t>(c) * taps : nullptr;
     // the normed value of portion row k of this channel (k < 0: from the carried state, or zero)
@@ -122,6 +129,96 @@ __global__ __launch_bounds__(kNormThreads) void norm_conv_kernel(hymeta_norm_con
       // new state row r = the normed row at portion index q - hist + r; indices before the portion come from the old
       // state (row q + r, which lies after the row being written: ascending r never reads a row already replaced)
       for (int r = 0; r < hist; ++r) A::st(state + static_cast<int64_t>(r) * a.width + c, normed(q - hist + r));
+    }
+  };
+#pragma unroll
+  for (int u = 0; u < kRowUnroll; ++u) {
+    const int c = threadIdx.x + u * kNormThreads;
+    if (c < a.width) emit_at(c);
+  }
+  for (int c = threadIdx.x + kRowUnroll * kNormThreads; c < a.width; c += kNormThreads) emit_at(c);
+}
+
+// Sequence of row t, with the shortcut for steps of single rows (sequence t at row t).
+__device__ __forceinline__ int seq_of_row_fast(const hymeta_norm_conv_args& a, int t) {
+  if (t < a.num_seqs && a.query_start_loc[t] == t && a.query_start_loc[t + 1] == t + 1) return t;
+  return seq_of_row(a.query_start_loc, a.num_seqs, t);
+}
+
+constexpr int kStripHist = 3;                  // the strip form covers taps <= 4 ...
+constexpr int kStripPerThread = 16;            // ... and width <= 256 * 16
+
+// A workgroup per strip of R consecutive rows.  Where the strip lies inside one portion, past the rows that read the
+// carried state, its R + taps - 1 input rows are read once into registers, their statistics reduced together, and every
+// output row takes its predecessors from the registers; other strips (a portion's first rows, strips over a boundary
+// between sequences) go row by row through norm_conv_row.
+template <typename A, int R>
+__global__ __launch_bounds__(kNormThreads) void norm_conv_kernel(hymeta_norm_conv_args a) {
+  typedef typename A::elem elem;
+  __shared__ float red[kNormWaves][kMaxRows];
+  const int t0 = blockIdx.x * R;
+  const int rows = min(R, a.num_tokens - t0);
+  const int taps = a.conv_weight ? a.taps : 1;
+  const int hist = taps - 1;
+  bool strip = false;
+  if (R > 1 && hist > 0 && hist <= kStripHist && rows == R && a.width <= kNormThreads * kStripPerThread) {
+    const int s0 = seq_of_row_fast(a, t0);
+    strip = t0 - a.query_start_loc[s0] >= hist && t0 + R <= a.query_start_loc[s0 + 1];
+  }
+  if (!strip) {
+    for (int r = 0; r < rows; ++r) {
+      norm_conv_row<A>(a, t0 + r, red);
+      __syncthreads();                         // red is reused by the next row
+    }
+    return;
+  }
+  // register image: input row t0 + R - 1 - m at v[m], m < R + hist (every index below is a compile-time constant)
+  constexpr int kIn = R + kStripHist;
+  float v[kIn][kStripPerThread];
+  float ss[kIn];
+#pragma unroll
+  for (int m = 0; m < kIn; ++m) {
+    ss[m] = 0.f;
+    const bool used = m < R + hist;
+    const float* row = a.x + (static_cast<int64_t>(t0) + R - 1 - m) * a.x_stride_t;
+#pragma unroll
+    for (int u = 0; u < kStripPerThread; ++u) {
+      const int c = threadIdx.x + u * kNormThreads;
+      v[m][u] = (used && c < a.width) ? row[c] : 0.f;
+      ss[m] = fmaf(v[m][u], v[m][u], ss[m]);
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < kIn; ++m) {
+    const float w = wave_sum(ss[m]);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6][m] = w;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int m = 0; m < kIn; ++m) {
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < kNormWaves; ++w) tot += red[w][m];
+    const float inv = 1.f / sqrtf(tot / static_cast<float>(a.width) + a.eps);
+#pragma unroll
+    for (int u = 0; u < kStripPerThread; ++u) {
+      const int c = threadIdx.x + u * kNormThreads;
+      v[m][u] = c < a.width ? A::round(v[m][u] * inv * (a.weight_offset + a.weight[c])) : 0.f;
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kStripPerThread; ++u) {
+    const int c = threadIdx.x + u * kNormThreads;
+    if (c >= a.width) continue;
+    float back[kStripHist + 1];                 // the tap that reads the row d steps back (d = 0: the row itself)
+#pragma unroll
+    for (int d = 0; d <= kStripHist; ++d) back[d] = d <= hist ? a.conv_weight[static_cast<int64_t>(c) * taps + hist - d] : 0.f;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float acc = v[R - 1 - r][u];
+#pragma unroll
+      for (int d = kStripHist; d >= 0; --d) acc = fmaf(back[d], v[R - 1 - r + d][u], acc);     // oldest row first, as the row form
+      A::st(static_cast<elem*>(a.out) + (static_cast<int64_t>(t0) + r) * a.width + c, acc);
     }
   }
 }
@@ -185,8 +282,16 @@ extern "C" int hymeta_norm_conv(const hymeta_norm_conv_args* args, hymeta_stream
     if (a.taps > 1 && (a.num_seqs <= 0 || !a.query_start_loc || !a.context_lens)) return HYMETA_ERR_INVALID_ARG;
   }
   hipStream_t st = begin_launches(stream);
-  if (a.act_dtype == HYMETA_BF16) hipLaunchKernelGGL(norm_conv_kernel<ActBf16>, dim3(a.num_tokens), dim3(kNormThreads), 0, st, a);
-  else hipLaunchKernelGGL(norm_conv_kernel<ActF32>, dim3(a.num_tokens), dim3(kNormThreads), 0, st, a);
+  // many rows: strips of four (their inputs read once); few rows (decode): a workgroup per row
+  const bool strips = a.num_tokens >= 1024 && a.conv_weight != nullptr && a.taps > 1;
+  const dim3 grid(strips ? (a.num_tokens + 3) / 4 : a.num_tokens);
+  if (a.act_dtype == HYMETA_BF16) {
+    if (strips) hipLaunchKernelGGL((norm_conv_kernel<ActBf16, 4>), grid, dim3(kNormThreads), 0, st, a);
+    else hipLaunchKernelGGL((norm_conv_kernel<ActBf16, 1>), grid, dim3(kNormThreads), 0, st, a);
+  } else {
+    if (strips) hipLaunchKernelGGL((norm_conv_kernel<ActF32, 4>), grid, dim3(kNormThreads), 0, st, a);
+    else hipLaunchKernelGGL((norm_conv_kernel<ActF32, 1>), grid, dim3(kNormThreads), 0, st, a);
+  }
   return launch_status();
 }
 

@@ -175,21 +175,45 @@ struct TileStage {
   u32x4 rk[kKeyPerThread];
   u32x4 rv[4];
 
-  static __device__ __forceinline__ const uint16_t* row_ptr(const hymeta_sink_attention_args& a, const int32_t* bt, int g, int j) {
-    // pages hold a power of two of rows here (the host sends other sizes to the plain kernel): shift and mask
-    const int page_shift = __builtin_ctz(a.block_size), page_mask = a.block_size - 1;
-    const int64_t blk = bt[j >> page_shift];
-    return static_cast<const uint16_t*>(a.kv_cache) +
-           ((blk << page_shift) + (j & page_mask)) * (static_cast<int64_t>(a.num_kv_heads) * (D + DV)) + static_cast<int64_t>(g) * (D + DV);
+  // Pages hold a power of two of rows here (the host sends other sizes to the plain kernel).  A page of 64 rows or more
+  // holds a whole tile (tiles start at multiples of 64): its number is one scalar load per tile, not a dependent vector
+  // load in front of every row's loads.
+  struct Pages {
+    const uint16_t* cache;
+    const int32_t* bt;
+    int64_t row_elems, head_off;
+    int shift, mask;
+    int64_t tile_base;          // first row of the tile's page, in rows of the cache (pages of >= 64 rows)
+    bool whole;
+  };
+
+  static __device__ __forceinline__ Pages pages(const hymeta_sink_attention_args& a, const int32_t* bt, int g, int j0) {
+    Pages p;
+    p.cache = static_cast<const uint16_t*>(a.kv_cache);
+    p.bt = bt;
+    p.row_elems = static_cast<int64_t>(a.num_kv_heads) * (D + DV);
+    p.head_off = static_cast<int64_t>(g) * (D + DV);
+    p.shift = __builtin_ctz(a.block_size);
+    p.mask = a.block_size - 1;
+    p.whole = a.block_size >= kTileKeys;
+    p.tile_base = 0;
+    if (p.whole) p.tile_base = (static_cast<int64_t>(__builtin_amdgcn_readfirstlane(bt[j0 >> p.shift])) << p.shift) + (j0 & p.mask);
+    return p;
+  }
+
+  static __device__ __forceinline__ const uint16_t* row_ptr(const Pages& p, int j0, int j) {
+    const int64_t row = p.whole ? p.tile_base + (j - j0) : (static_cast<int64_t>(p.bt[j >> p.shift]) << p.shift) + (j & p.mask);
+    return p.cache + row * p.row_elems + p.head_off;
   }
 
   __device__ __forceinline__ void issue(const hymeta_sink_attention_args& a, const int32_t* bt, int g, int j0, int last) {
+    const Pages p = pages(a, bt, g, j0);
 #pragma unroll
     for (int i = 0; i < kKeyPerThread; ++i) {
       const int idx = i * Threads + threadIdx.x;
       const int j = j0 + idx / kKeyChunksPerRow;
       rk[i] = u32x4{0u, 0u, 0u, 0u};
-      if (j <= last) rk[i] = ld16g(row_ptr(a, bt, g, j) + (idx % kKeyChunksPerRow) * 8);
+      if (j <= last) rk[i] = ld16g(row_ptr(p, j0, j) + (idx % kKeyChunksPerRow) * 8);
     }
     if (static_cast<int>(threadIdx.x) < kValBlocks) {
       const int ch = threadIdx.x % kValChunksPerRow, grp = threadIdx.x / kValChunksPerRow;
@@ -197,7 +221,7 @@ struct TileStage {
       for (int i = 0; i < 4; ++i) {
         const int j = j0 + 4 * grp + i;
         rv[i] = u32x4{0u, 0u, 0u, 0u};
-        if (j <= last) rv[i] = ld16g(row_ptr(a, bt, g, j) + D + ch * 8);
+        if (j <= last) rv[i] = ld16g(row_ptr(p, j0, j) + D + ch * 8);
       }
     }
   }
@@ -356,7 +380,7 @@ constexpr int kPrefillRows = 16 * kPrefillWaves;
 // Portions of prompts: grid = (tiles of 128 rows, heads, sequences); sequences with one row are left to the decode form.
 template <int D, int DV>
 __global__ __launch_bounds__(64 * kPrefillWaves) void sink_attention_prefill_mfma_kernel(hymeta_sink_attention_args a) {
-  __shared__ MfmaSmem<D, DV> sm;
+  __shared__ MfmaSmem<D, DV> sm[2];
   const int s = blockIdx.z, h = blockIdx.y;
   const int row0 = a.query_start_loc[s];
   const int q = a.query_start_loc[s + 1] - row0;
@@ -381,14 +405,19 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void sink_attention_prefill_mfm
   const int wave_last = ctx + min(q, wrow + 16) - 1;
   int j_first = 0;
   if (a.window_left >= 0) j_first = max(0, ctx + static_cast<int>(blockIdx.x) * kPrefillRows - a.window_left) / kTileKeys * kTileKeys;
+  // two LDS images: while the waves multiply tile t out of one, tile t + 1 goes into the other and the loads of tile
+  // t + 2 are in flight; one barrier per tile
   TileStage<D, DV, 64 * kPrefillWaves> stage;
   stage.issue(a, bt, g, j_first, block_last);
-  for (int j0 = j_first; j0 <= block_last; j0 += kTileKeys) {
-    __syncthreads();                   // every wave is done with the tile before
-    stage.commit(sm);
+  stage.commit(sm[0]);
+  if (j_first + kTileKeys <= block_last) stage.issue(a, bt, g, j_first + kTileKeys, block_last);
+  __syncthreads();
+  int buf = 0;
+  for (int j0 = j_first; j0 <= block_last; j0 += kTileKeys, buf ^= 1) {
+    if (j0 + kTileKeys <= block_last) stage.commit(sm[buf ^ 1]);
+    if (j0 + 2 * kTileKeys <= block_last) stage.issue(a, bt, g, j0 + 2 * kTileKeys, block_last);
+    if (wrow < q && j0 <= wave_last) attend_tile<D, DV, 1, 4>(w, sm[buf], a, j0, 0);
     __syncthreads();
-    if (j0 + kTileKeys <= block_last) stage.issue(a, bt, g, j0 + kTileKeys, block_last);
-    if (wrow < q && j0 <= wave_last) attend_tile<D, DV, 1, 4>(w, sm, a, j0, 0);
   }
   if (!ok) return;
   float l = w.l[0];
@@ -413,7 +442,7 @@ constexpr int kDecodeWaves = 4;
 // weighted values) per head; the combine kernel merges them and the sink.
 template <int D, int DV, int RB>
 __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_kernel(hymeta_sink_attention_args a, int splits, int tiles_per_split) {
-  __shared__ MfmaSmem<D, DV> sm;
+  __shared__ MfmaSmem<D, DV> sm[2];
   const int s = blockIdx.z, g = blockIdx.y, split = blockIdx.x;
   const int t = a.query_start_loc[s];
   if (a.query_start_loc[s + 1] - t != 1) return;
@@ -444,13 +473,18 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
   }
   if (j_lo < first) j_lo = first / kTileKeys * kTileKeys;      // tiles wholly before the window are not read
   TileStage<D, DV, 64 * kDecodeWaves> stage;
-  if (j_lo <= j_hi) stage.issue(a, bt, g, j_lo, j_hi);
-  for (int j0 = j_lo; j0 <= j_hi; j0 += kTileKeys) {
+  if (j_lo <= j_hi) {
+    stage.issue(a, bt, g, j_lo, j_hi);
+    stage.commit(sm[0]);
+    if (j_lo + kTileKeys <= j_hi) stage.issue(a, bt, g, j_lo + kTileKeys, j_hi);
+  }
+  __syncthreads();
+  int buf = 0;
+  for (int j0 = j_lo; j0 <= j_hi; j0 += kTileKeys, buf ^= 1) {
+    if (j0 + kTileKeys <= j_hi) stage.commit(sm[buf ^ 1]);
+    if (j0 + 2 * kTileKeys <= j_hi) stage.issue(a, bt, g, j0 + 2 * kTileKeys, j_hi);
+    if (j0 + 16 * wave <= j_hi) attend_tile<D, DV, RB, 1>(w, sm[buf], a, j0, wave);
     __syncthreads();
-    stage.commit(sm);
-    __syncthreads();
-    if (j0 + kTileKeys <= j_hi) stage.issue(a, bt, g, j0 + kTileKeys, j_hi);
-    if (j0 + 16 * wave <= j_hi) attend_tile<D, DV, RB, 1>(w, sm, a, j0, wave);
   }
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
