@@ -1130,9 +1130,13 @@ typedef struct hymeta_mingru_args {
   const int32_t* query_start_loc;
   const int32_t* context_lens;
   const int32_t* slot_idx;
-  int32_t num_tokens, num_seqs, width, act_dtype, max_query_len;
+  int32_t num_tokens, num_seqs, width, act_dtype, max_query_len;   /* max_query_len: upper bound of the portions' rows */
   int64_t zug_stride_t;
+  void* workspace;             /* hymeta_mingru_workspace_bytes(num_seqs, width, max_query_len) bytes, or NULL when that is 0 */
+  size_t workspace_bytes;
 } hymeta_mingru_args;
+/* > 0 for steps with long portions: they are scanned in segments that run side by side (three launches). */
+size_t hymeta_mingru_workspace_bytes(int32_t num_seqs, int32_t width, int32_t max_query_len);
 int hymeta_mingru(const hymeta_mingru_args* args, hymeta_stream_t stream);
 
 /* Per-head RMS norm of the query and key columns of a fused q|k|v projection and the paged write of

@@ -140,6 +140,30 @@ def test_mingru_prefill_equals_token_by_token_and_portions(dtype, width):
         assert float(state[0].min()) == 5.0 and float(state[2].max()) == 5.0      # other slots untouched
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mingru_long_portions_run_in_segments(dtype):
+    """Portions of thousands of rows are scanned in segments side by side and chained; a short sequence shares the step, and
+    the long one goes on from the state a first portion left."""
+    from vllm_hymeta import hip_ops
+    g = torch.Generator().manual_seed(21)
+    width, T, first = 72, 2400, 37
+    zug, short = bf16_values(T, 3 * width, std=1.5, gen=g), bf16_values(5, 3 * width, gen=g)
+    eye, zero = torch.eye(width, dtype=torch.float64), torch.zeros(width, width, dtype=torch.float64)
+    pick = [torch.cat([eye if j == n else zero for j in range(3)], 1) for n in range(3)]
+    none = torch.zeros(width).double()
+    ref, ref_short = mingru_ref(zug, pick[0], none, pick[1], none, pick[2], eye), mingru_ref(short, pick[0], none, pick[1], none, pick[2], eye)
+    state = torch.full((3, width), 9.0, dtype=torch.float32, device=DEV)
+    zd = zug.to(dtype).to(DEV)
+    a = hip_ops.mingru(zd[:first], state, i32([0, first]), i32([0]), i32([2]), first)
+    rows = torch.cat([short.to(dtype).to(DEV), zd[first:]])
+    b = hip_ops.mingru(rows, state, i32([0, 5, 5 + T - first]), i32([0, first]), i32([0, 2]), T - first)
+    assert rel_err(torch.cat([a, b[5:]]), ref) < TOL[dtype]
+    assert rel_err(b[:5], ref_short) < TOL[dtype]
+    whole = hip_ops.mingru(zd, state, i32([0, T]), i32([0]), i32([1]), T)
+    assert rel_err(whole, ref) < TOL[dtype]
+    assert rel_err(state[1], state[2]) < 1e-5        # the same final state whichever way the rows were cut
+
+
 def test_mingru_batches_unequal_sequences():
     from vllm_hymeta import hip_ops
     g = torch.Generator().manual_seed(9)

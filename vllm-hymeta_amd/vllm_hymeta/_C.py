@@ -326,7 +326,7 @@ class MinGruArgs(_Args):
         ("zug", _ptr), ("state", _ptr), ("out", _ptr),
         ("query_start_loc", _ptr), ("context_lens", _ptr), ("slot_idx", _ptr),
         ("num_tokens", _i32), ("num_seqs", _i32), ("width", _i32), ("act_dtype", _i32), ("max_query_len", _i32),
-        ("zug_stride_t", _i64),
+        ("zug_stride_t", _i64), ("workspace", _ptr), ("workspace_bytes", _sz),
     ]
 
 
@@ -453,6 +453,7 @@ _SIGNATURES = {
     "hymeta_embed_rows": (C.c_int, [C.POINTER(EmbedRowsArgs), _ptr]),
     "hymeta_norm_conv": (C.c_int, [C.POINTER(NormConvArgs), _ptr]),
     "hymeta_norm_residual": (C.c_int, [C.POINTER(NormResidualArgs), _ptr]),
+    "hymeta_mingru_workspace_bytes": (_sz, [_i32, _i32, _i32]),
     "hymeta_mingru": (C.c_int, [C.POINTER(MinGruArgs), _ptr]),
     "hymeta_qk_norm_cache": (C.c_int, [C.POINTER(QkNormCacheArgs), _ptr]),
     "hymeta_sink_attention_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32, _i32]),

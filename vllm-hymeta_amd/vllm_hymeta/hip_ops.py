@@ -1564,7 +1564,12 @@ def mingru(zug: torch.Tensor, state: torch.Tensor, query_start_loc: torch.Tensor
     a.zug, a.state, a.out = _p(zug), _p(state), _p(out)
     a.query_start_loc, a.context_lens, a.slot_idx = _p(query_start_loc), _p(context_lens), _p(slot_idx)
     a.num_tokens, a.num_seqs, a.width, a.act_dtype, a.max_query_len, a.zug_stride_t = T, S, W, _act(zug), max_query_len, zug.stride(0)
-    _C.check(_C.load().hymeta_mingru(C.byref(a), _stream(zug)), "hymeta_mingru")
+    lib = _C.load()
+    nbytes = int(lib.hymeta_mingru_workspace_bytes(S, W, max_query_len))
+    if nbytes:
+        ws = _workspace(zug.device, nbytes, "mingru")
+        a.workspace, a.workspace_bytes = _p(ws), ws.numel()
+    _C.check(lib.hymeta_mingru(C.byref(a), _stream(zug)), "hymeta_mingru")
     return out
 
 
