@@ -101,3 +101,14 @@ def test_oracle_is_causal_and_its_mechanisms_show_in_the_logits():
     cw = torch.tensor([[1.0, 0.0], [0.0, 1.0], [2.0, 3.0]], dtype=torch.float64)
     out = causal_conv_add_ref(h, cw)
     assert out[0].tolist() == [0.0, 2.0, 8.0] and out[2].tolist() == [6 + 3, 7 + 7, 8 + 2 * 5 + 3 * 8]
+
+
+def test_registry_names_the_kernel_sources_the_model_class_names():
+    """The table a first run reads before torch is imported says what the class says, and every name is a source file."""
+    import os
+    from vllm_hymeta import registry
+    from vllm_hymeta.models.modeling_sonuzen import SonuzenForCausalLM
+    assert registry._KERNEL_SOURCES["SonuzenForCausalLM"] == SonuzenForCausalLM.kernel_sources
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "vllm-hymeta_amd", "csrc")
+    for name in SonuzenForCausalLM.kernel_sources:
+        assert os.path.exists(os.path.join(csrc, name + ".hip")), name

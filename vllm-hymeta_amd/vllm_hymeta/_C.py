@@ -494,6 +494,35 @@ STRUCTS = {
 }
 
 
+_missing: list = []
+
+
+def missing_symbols():
+    """Declared symbols the loaded library does not export (empty for a complete build)."""
+    return list(_missing)
+
+
+def _absent_symbol(name: str, path: str):
+    def call(*_args, **_kwargs):
+        raise HymetaError(f"{name} is not in {path}: the library was linked from a part of the sources; "
+                          "run `make -C vllm-hymeta_amd` to complete it")
+    return call
+
+
+def build_library(sources=None) -> None:
+    """Compile the library in-tree with the Makefile: every source, or (``sources``: stems of ``csrc/*.hip``) the part a
+    model needs.  Called where a fresh checkout is about to run for the first time; an existing library is left alone."""
+    import subprocess
+    import sys
+    if os.path.exists(library_path()):
+        return
+    pkg = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cmd = ["make", "-C", pkg, f"-j{min(16, os.cpu_count() or 1)}"]
+    if sources:
+        cmd.append("ONLY=" + " ".join(sources))
+    subprocess.run(cmd, check=True, stdout=sys.stderr, stderr=sys.stderr)
+
+
 def library_path() -> str:
     return os.environ.get("HYMETA_HIP_LIB") or os.path.join(
         os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
@@ -519,10 +548,20 @@ def load() -> C.CDLL:
     import torch  # noqa: F401
 
     lib = C.CDLL(path)
+    absent = []
     for name, (restype, argtypes) in _SIGNATURES.items():
-        fn = getattr(lib, name)  # AttributeError names the missing symbol
+        try:
+            fn = getattr(lib, name)
+        except AttributeError:
+            # a library linked from a part of the sources (``make ONLY=...``, see ``build_library``): the call raises
+            absent.append(name)
+            setattr(lib, name, _absent_symbol(name, path))
+            continue
         fn.restype = restype
         fn.argtypes = argtypes
+    if "hymeta_abi_version" in absent or len(absent) == len(_SIGNATURES):
+        raise RuntimeError(f"{path} exports none of the declared symbols")
+    _missing[:] = absent
     version = lib.hymeta_abi_version()
     if version != ABI_VERSION:
         raise RuntimeError(f"{path}: ABI version {version}, binding expects {ABI_VERSION}")

@@ -136,6 +136,9 @@ class SonuzenModel(torch.nn.Module):
 
 
 class SonuzenForCausalLM(torch.nn.Module, HasInnerState, IsHybrid):
+    # csrc/*.hip sources whose kernels this class calls (a first run in a fresh checkout builds these, see _C.build_library)
+    kernel_sources = ("api_misc", "norm_conv", "mingru", "sink_attn", "moe_table", "moe", "glue", "dense_gemm", "stream_gemm", "tall_gemm")
+
     def __init__(self, config: Optional[SonuzenConfig] = None, max_num_seqs: int = 256, dtype: torch.dtype = torch.bfloat16,
                  device="cuda", *, vllm_config=None, prefix: Optional[str] = None):
         super().__init__()

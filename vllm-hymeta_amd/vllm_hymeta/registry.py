@@ -50,5 +50,18 @@ def resolve(model_dir: str):
     return getattr(importlib.import_module(module), name), load_config(model_dir)
 
 
+def kernel_sources(model_dir: str):
+    """The kernel sources the checkpoint's model class names (None: the whole library), read without importing torch."""
+    path, _ = _MODELS[architecture_of(model_dir)]
+    return _KERNEL_SOURCES.get(path.partition(":")[2])
+
+
+# (kept beside the table so that asking does not import the model module, which imports torch and the library binding)
+_KERNEL_SOURCES = {
+    "SonuzenForCausalLM": ("api_misc", "norm_conv", "mingru", "sink_attn", "moe_table", "moe", "glue", "dense_gemm", "stream_gemm",
+                           "tall_gemm"),
+}
+
+
 def known_architectures():
     return sorted(_MODELS)
