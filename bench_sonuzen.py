@@ -80,7 +80,7 @@ def sonuzen_checkpoint(cfg, dev, seed=0):
             yield f"{p}mlp.e{e}.gate", rnd(ff, W, std=W ** -0.5)
             yield f"{p}mlp.e{e}.up", rnd(ff, W, std=W ** -0.5)
             yield f"{p}mlp.e{e}.down", rnd(W, ff, std=ff ** -0.5)
-        yield p + "mlp.table", torch.stack([torch.randperm(E, device=dev, generator=g)[:top] for _ in range(V)]).to(torch.int32)
+        yield p + "mlp.table", torch.rand(V, E, device=dev, generator=g).argsort(1)[:, :top].to(torch.int32).contiguous()
 
 
 class SonuzenRunner:
@@ -260,7 +260,7 @@ def kernel_table(dev, W, H, G, D, B, ctx, L, E, top, ff):
         add(f"add_rmsnorm (7B) T={T}", lambda: hip_ops.add_rmsnorm(xb, w7, 1e-6, residual=res), nbytes=T * W * (2 + 2 + 2 + 2))
     # ---- experts
     w13, w2 = rnd(E, 2 * ff, W, std=W ** -0.5), rnd(E, W, ff, std=ff ** -0.5)
-    table = torch.stack([torch.randperm(E, device=dev)[:top] for _ in range(1024)]).to(torch.int32)
+    table = torch.rand(1024, E, device=dev).argsort(1)[:, :top].to(torch.int32).contiguous()
     for T in (B, L):
         xm = rnd(T, W)
         ids = torch.randint(0, 1024, (T,), device=dev)

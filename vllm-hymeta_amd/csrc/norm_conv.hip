@@ -165,6 +165,64 @@ __global__ __launch_bounds__(kNormThreads) void norm_conv_kernel(hymeta_norm_con
     const int s0 = seq_of_row_fast(a, t0);
     strip = t0 - a.query_start_loc[s0] >= hist && t0 + R <= a.query_start_loc[s0 + 1];
   }
+  if (R == 1 && hist <= kStripHist && a.width <= kNormThreads * kStripPerThread) {
+    // a sequence's only row in this step (every row of a decode step; every row when there is no convolution): the row,
+    // its predecessors from the carried state, and the state's shift, without a branch between the loads
+    int q = 1, ctx = 0, slot = -1;
+    if (hist > 0) {
+      const int s = seq_of_row_fast(a, t0);
+      q = a.query_start_loc[s + 1] - a.query_start_loc[s];
+      ctx = a.context_lens[s];
+      slot = a.slot_idx ? a.slot_idx[s] : -1;
+    }
+    if (q == 1) {
+      elem* state = (hist > 0 && a.conv_state && slot >= 0) ? static_cast<elem*>(a.conv_state) + static_cast<int64_t>(slot) * hist * a.width
+                                                            : nullptr;
+      const bool carried = state != nullptr && ctx > 0;
+      const float* row = a.x + static_cast<int64_t>(t0) * a.x_stride_t;
+      float x[kStripPerThread], back[kStripHist][kStripPerThread];     // back[d - 1]: the normed row d steps back
+      float ss = 0.f;
+#pragma unroll
+      for (int u = 0; u < kStripPerThread; ++u) {
+        const int c = threadIdx.x + u * kNormThreads;
+        x[u] = c < a.width ? row[c] : 0.f;
+        ss = fmaf(x[u], x[u], ss);
+#pragma unroll
+        for (int d = 1; d <= kStripHist; ++d)
+          back[d - 1][u] = (carried && d <= hist && c < a.width) ? A::ld(state + static_cast<int64_t>(hist - d) * a.width + c) : 0.f;
+      }
+      ss = wave_sum(ss);
+      if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6][0] = ss;
+      __syncthreads();
+      float tot = 0.f;
+#pragma unroll
+      for (int w = 0; w < kNormWaves; ++w) tot += red[w][0];
+      const float inv = 1.f / sqrtf(tot / static_cast<float>(a.width) + a.eps);
+#pragma unroll
+      for (int u = 0; u < kStripPerThread; ++u) {
+        const int c = threadIdx.x + u * kNormThreads;
+        if (c >= a.width) continue;
+        const float n = A::round(x[u] * inv * (a.weight_offset + a.weight[c]));
+        float acc = n;
+        if (a.conv_weight != nullptr) {
+          const float* cw = a.conv_weight + static_cast<int64_t>(c) * taps;
+          acc = fmaf(cw[hist], n, acc);
+#pragma unroll
+          for (int d = kStripHist; d >= 1; --d)
+            if (d <= hist) acc = fmaf(cw[hist - d], back[d - 1][u], acc);
+        }
+        A::st(static_cast<elem*>(a.out) + static_cast<int64_t>(t0) * a.width + c, acc);
+        if (state != nullptr) {
+          // the state moves up one row: the row d steps back goes to row hist - 1 - d, this row to the last
+          A::st(state + static_cast<int64_t>(hist - 1) * a.width + c, n);
+#pragma unroll
+          for (int d = 1; d < kStripHist; ++d)
+            if (d <= hist - 1) A::st(state + static_cast<int64_t>(hist - 1 - d) * a.width + c, back[d - 1][u]);
+        }
+      }
+      return;
+    }
+  }
   if (!strip) {
     for (int r = 0; r < rows; ++r) {
       norm_conv_row<A>(a, t0 + r, red);
