@@ -1671,7 +1671,7 @@ def moe_table_forward(x: torch.Tensor, token_ids: torch.Tensor, table: torch.Ten
     r.num_tokens, r.num_experts, r.top_k, r.vocab = T, E, top, table.shape[0]
     _C.check(lib.hymeta_moe_route_table(C.byref(r), st), "hymeta_moe_route_table")
 
-    if (x.dtype == torch.bfloat16 and moe_mfma_shapes(H, inter) and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
+    if (x.dtype == torch.bfloat16 and moe_mfma_shapes(H, inter) and E <= 64 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
         h13 = torch.empty(P, two_i, dtype=torch.bfloat16, device=dev)
         g = _C.MoeGemmArgs()
         g.x, g.weights, g.out, g.expert_offsets = _p(x), _p(w13), _p(h13), _p(offsets)
