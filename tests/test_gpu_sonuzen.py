@@ -308,7 +308,7 @@ def build_engine(cfg, weights, dtype, max_tokens=512, block_size=16, max_num_seq
 
 
 MODELS = {
-    "hybrid_loop": dict(layers=("attention", "attention", "mingru", "attention"), loop=(1, 3, 2)),
+    "hybrid_loop": dict(layers=("mingru", "attention", "attention", "mingru", "attention"), loop=(1, 4, 2)),
     "loop_from_first_layer_three_times": dict(layers=("mingru", "attention"), loop=(0, 2, 3), taps=2, top=1, experts=3),
     "no_loop_wide_gru_no_mlp_on_one": dict(layers=("attention", "mingru", "mingru"), mingru_width=96, no_mlp=(1,), taps=4,
                                            heads=6, kv_heads=3, dim=8, vdim=8, top=3, experts=5, ff=24, width=48, residual_mult=1.0,
