@@ -278,7 +278,7 @@ struct WaveRows {
 
 typedef short bf16x4 __attribute__((ext_vector_type(4)));
 
-template <int D, int DV, int RB, int NKS>
+template <int D, int DV, int RB, int NKS, bool Masked>
 __device__ __forceinline__ void attend_tile(WaveRows<D, DV, RB>& w, const MfmaSmem<D, DV>& sm, const hymeta_sink_attention_args& a,
                                             int j0, int ks_lo) {
   static_assert(NKS == 4 || NKS == 1, "all of a tile's subtiles or one");
@@ -297,43 +297,53 @@ __device__ __forceinline__ void attend_tile(WaveRows<D, DV, RB>& w, const MfmaSm
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) s[rb][ks] = mfma16(kf, w.q[rb][st], s[rb][ks]);
     }
-  // lane holds, per row block, the scores of its row (n) against keys j0 + 16 (ks_lo + ks) + 4 g4 + r
+  // lane holds, per row block, the scores of its row (n) against keys j0 + 16 (ks_lo + ks) + 4 g4 + r.  Everything from
+  // here to the weights is in the base-2 domain (scores times log2 e; the bias' coefficient is unchanged, as
+  // a ln x * log2 e = a log2 x): one v_log and one v_exp per score and no multiplications around them.  The running
+  // maximum, and with it the sink's score 0, mean the same in both domains.
+  const float scale2 = a.scale * 1.4426950408889634f;
+  const bool bias = a.bias_mode == HYMETA_BIAS_LOG_DISTANCE;
   uint32_t phi[RB][NKS][2], plo[RB][NKS][2];       // the weights' bf16 high and low parts, two per dword
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int pos = w.pos[rb];
-    const int first = a.window_left >= 0 ? pos - a.window_left : 0;
+    // distance of the lane's key r of subtile ks: fd0 - (16 ks + r)
+    const float fd0 = static_cast<float>(pos - j0 - 16 * ks_lo - 4 * g4);
     float mx = -INFINITY;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int j = j0 + 16 * (ks_lo + ks) + 4 * g4 + r;
-        float sc = s[rb][ks][r] * a.scale;
-        if (a.bias_mode == HYMETA_BIAS_LOG_DISTANCE) sc -= w.ba[rb] * __logf(1.f + w.bb[rb] * static_cast<float>(pos - j));
-        sc = (j <= pos && j >= first) ? sc : -INFINITY;
+        float sc = s[rb][ks][r] * scale2;
+        if (bias) sc = fmaf(-w.ba[rb], __log2f(fmaf(w.bb[rb], fd0 - static_cast<float>(16 * ks + r), 1.f)), sc);
+        if (Masked) {
+          const int j = j0 + 16 * (ks_lo + ks) + 4 * g4 + r;
+          const int first = a.window_left >= 0 ? pos - a.window_left : 0;
+          sc = (j <= pos && j >= first) ? sc : -INFINITY;
+        }
         s[rb][ks][r] = sc;
         mx = fmaxf(mx, sc);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(w.m[rb], mx);
-    // a row with nothing visible so far and no sink keeps m = -inf: every weight and the correction are then 0
-    const float corr = m_new == -INFINITY ? 0.f : __expf(w.m[rb] - m_new);
+    // (masked tiles only) a row with nothing visible so far and no sink keeps m = -inf: weights and correction are 0
+    const bool empty = Masked && m_new == -INFINITY;
+    const float corr = empty ? 0.f : __builtin_amdgcn_exp2f(w.m[rb] - m_new);
     float sum = 0.f;
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks)
 #pragma unroll
       for (int r2 = 0; r2 < 2; ++r2) {
-        float p[2], res[2];
+        float p[2];
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-          p[u] = m_new == -INFINITY ? 0.f : __expf(s[rb][ks][2 * r2 + u] - m_new);
+          p[u] = empty ? 0.f : __builtin_amdgcn_exp2f(s[rb][ks][2 * r2 + u] - m_new);
           sum += p[u];
-          res[u] = p[u] - bf16_round(p[u]);
         }
-        phi[rb][ks][r2] = pack_bf16x2(p[0], p[1]);
-        plo[rb][ks][r2] = pack_bf16x2(res[0], res[1]);
+        const uint32_t hi = pack_bf16x2(p[0], p[1]);
+        phi[rb][ks][r2] = hi;
+        plo[rb][ks][r2] = pack_bf16x2(p[0] - lo_bf(hi), p[1] - hi_bf(hi));
       }
     w.l[rb] = w.l[rb] * corr + sum;
     w.m[rb] = m_new;
@@ -427,7 +437,11 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void sink_attention_prefill_mfm
   for (int j0 = j_first; j0 <= block_last; j0 += kTileKeys, buf ^= 1) {
     if (j0 + kTileKeys <= block_last) stage.commit(sm[buf ^ 1]);
     if (j0 + 2 * kTileKeys <= block_last) stage.issue(a, bt, g, j0 + 2 * kTileKeys, block_last);
-    if (wrow < q && j0 <= wave_last) attend_tile<D, DV, RB, 4>(w, sm[buf], a, j0, 0);
+    if (wrow < q && j0 <= wave_last) {
+      // tiles wholly before the wave's first row (and no window) need no mask: every key is visible to every row
+      if (a.window_left < 0 && j0 + kTileKeys - 1 <= ctx + wrow) attend_tile<D, DV, RB, 4, false>(w, sm[buf], a, j0, 0);
+      else attend_tile<D, DV, RB, 4, true>(w, sm[buf], a, j0, 0);
+    }
     __syncthreads();
   }
 #pragma unroll
@@ -498,7 +512,10 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
   for (int j0 = j_lo; j0 <= j_hi; j0 += kTileKeys, buf ^= 1) {
     if (j0 + kTileKeys <= j_hi) stage.commit(sm[buf ^ 1]);
     if (j0 + 2 * kTileKeys <= j_hi) stage.issue(a, bt, g, j0 + 2 * kTileKeys, j_hi);
-    if (j0 + 16 * wave <= j_hi) attend_tile<D, DV, RB, 1>(w, sm[buf], a, j0, wave);
+    if (j0 + 16 * wave <= j_hi) {
+      if (a.window_left < 0 && j0 + kTileKeys - 1 <= pos) attend_tile<D, DV, RB, 1, false>(w, sm[buf], a, j0, wave);
+      else attend_tile<D, DV, RB, 1, true>(w, sm[buf], a, j0, wave);
+    }
     __syncthreads();
   }
 #pragma unroll
@@ -526,12 +543,13 @@ __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymet
   const size_t stride = HG * partial_row_floats(DV);
   const float* base = static_cast<const float*>(a.workspace) + (static_cast<size_t>(s) * a.num_kv_heads + g) * splits * stride +
                       r * partial_row_floats(DV);
+  // (the partials' maxima are in the base-2 domain, as the waves kept them)
   float m = a.sink ? 0.f : -INFINITY;
   for (int sp = 0; sp < splits; ++sp) m = fmaxf(m, base[sp * stride + DV]);
-  float l = a.sink ? __expf(0.f - m) : 0.f;
+  float l = a.sink ? __builtin_amdgcn_exp2f(0.f - m) : 0.f;
   for (int sp = 0; sp < splits; ++sp) {
     const float ms = base[sp * stride + DV];
-    if (ms != -INFINITY) l += base[sp * stride + DV + 1] * __expf(ms - m);
+    if (ms != -INFINITY) l += base[sp * stride + DV + 1] * __builtin_amdgcn_exp2f(ms - m);
   }
   const float inv = l > 0.f ? 1.f / l : 0.f;
   uint16_t* out = static_cast<uint16_t*>(a.out) + (static_cast<int64_t>(t) * a.num_heads + h) * DV;
@@ -539,7 +557,7 @@ __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymet
     float acc = 0.f;
     for (int sp = 0; sp < splits; ++sp) {
       const float ms = base[sp * stride + DV];
-      if (ms != -INFINITY) acc += base[sp * stride + c] * __expf(ms - m);
+      if (ms != -INFINITY) acc += base[sp * stride + c] * __builtin_amdgcn_exp2f(ms - m);
     }
     out[c] = f2bf(acc * inv);
   }
