@@ -149,9 +149,9 @@ __device__ __forceinline__ f32x4v mfma16(bf16x8 a, bf16x8 b, f32x4v c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
-// Row blocks of 16 a prompt's wave holds.  Two halve the LDS reads per matrix instruction, but at 254 registers leave one
-// workgroup per compute unit, and the distance bias' logarithms are then no longer hidden: measured on an 8192-token
-// prompt (28 heads of 128) 3.0 ms against 2.55 ms with one (2.15 against 2.5 ms without the bias).
+// Row blocks of 16 a prompt's wave holds.  Two halve the LDS reads per matrix instruction, but at about 250 registers
+// leave one workgroup per compute unit: measured on prompts of 2048 / 4096 / 8192 rows (28 heads of 128) 0.20 / 0.59 /
+// 2.10 ms against 0.21 / 0.64 / 1.86 ms with one.
 #ifndef PREFILL_RB
 #define PREFILL_RB 1
 #endif
