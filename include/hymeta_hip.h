@@ -27,7 +27,9 @@
  *    with; a binding compares it with the header it was written against before
  *    the first call (version 2: every argument struct starts with struct_size;
  *    version 3: hymeta_gla_decode_args ends with qkv_x_scale / qkv_w_scale;
- *    version 4: the recurrent / biased-attention building blocks at the end of this file).
+ *    version 4: the recurrent / biased-attention building blocks;
+ *    version 5: hymeta_sink_attention_args ends with sink_logits / kv_layout, hymeta_moe_gemm_any_args with
+ *    act_limit / act_alpha; the post-norm, latent- and linear-attention building blocks at the end of this file).
  *  - Every argument struct starts with `uint32_t struct_size`, which the caller
  *    sets to sizeof(the struct) of ITS declaration.  An entry point returns
  *    HYMETA_ERR_INVALID_ARG, before it reads any other field, when the value
@@ -45,7 +47,7 @@
 extern "C" {
 #endif
 
-#define HYMETA_ABI_VERSION 4
+#define HYMETA_ABI_VERSION 5
 
 typedef void* hymeta_stream_t;
 
@@ -1162,7 +1164,8 @@ int hymeta_qk_norm_cache(const hymeta_qk_norm_cache_args* args, hymeta_stream_t 
  * the cache already), with a distance bias and an optional sink:
  *   s_ij = scale * q_i . k_j - bias(i - j),   j <= i   (and i - j <= window_left when window_left >= 0)
  *   bias_mode HYMETA_BIAS_NONE: 0;  HYMETA_BIAS_LOG_DISTANCE: bias_a[h] * ln(1 + bias_b[h] * (i - j))
- *   p_ij = exp(s_ij) / (sink + sum_j exp(s_ij)),  sink = 1 (a key of score 0 without a value) or 0
+ *   p_ij = exp(s_ij) / (sink + sum_j exp(s_ij)),  sink = exp(sink_logits[h]) (a key of that score, 0 without
+ *   sink_logits, that has no value and is neither scaled nor biased) or 0
  *   out_i = sum_j p_ij v_j
  * Scores and weights are fp32 in both activation types.  Query row t of sequence s stands at position
  * seq_lens[s] - (query_start_loc[s + 1] - t).  bf16 rows with head_dim and v_dim of 64 or 128 (and at
@@ -1172,6 +1175,12 @@ int hymeta_qk_norm_cache(const hymeta_qk_norm_cache_args* args, hymeta_stream_t 
  * max_query_len / max_seq_len: upper bounds of the step's portion and sequence lengths (they size the
  * grids).  Everything else runs a wave per (row, head). */
 enum hymeta_bias_mode { HYMETA_BIAS_NONE = 0, HYMETA_BIAS_LOG_DISTANCE = 1 };
+/* What a key/value head's part of a cache row holds.  KEY_THEN_VALUE: head_dim key elements followed by v_dim value
+ * elements (hymeta_qk_norm_cache).  VALUE_IN_KEY: head_dim elements, of which the first v_dim are also the value (a
+ * latent shared by keys and values followed by a rotated key part: hymeta_latent_kv_prep); v_dim <= head_dim.  With
+ * VALUE_IN_KEY bf16 rows of one key/value head, head_dim a multiple of 32 up to 576 and v_dim a multiple of 64 up to 512
+ * run on the matrix cores (rows = (token, head) pairs of a sequence, which all read the same key rows). */
+enum hymeta_kv_layout { HYMETA_KV_KEY_THEN_VALUE = 0, HYMETA_KV_VALUE_IN_KEY = 1 };
 typedef struct hymeta_sink_attention_args {
   uint32_t struct_size;
   const void* q;               /* act_dtype [num_tokens, num_heads, head_dim], strides q_stride_t / head_dim */
@@ -1188,6 +1197,8 @@ typedef struct hymeta_sink_attention_args {
   int32_t bias_mode, sink, window_left, max_query_len, max_seq_len;
   float scale;
   int64_t num_blocks, q_stride_t, block_table_stride;
+  const float* sink_logits;    /* [num_heads] or NULL: the sink's score per head (NULL: 0); read when sink != 0 */
+  int32_t kv_layout;           /* enum hymeta_kv_layout */
 } hymeta_sink_attention_args;
 size_t hymeta_sink_attention_workspace_bytes(int32_t num_seqs, int32_t num_heads, int32_t num_kv_heads, int32_t v_dim,
                                              int32_t max_seq_len);
@@ -1213,8 +1224,10 @@ int hymeta_moe_route_table(const hymeta_moe_route_table_args* args, hymeta_strea
 
 /* Grouped GEMM of the routed rows for any K and N and for fp32 or bf16 operands (hymeta_moe_gemm's
  * tiles need K % 32 == 0, N % 64 == 0 and bf16): out[slot] = x[row(slot)] W[e]^T, fp32 sums.
- * gated != 0: W[e] is [2 N, K] (gate rows, then up rows) and out[slot, n] = silu(gate_n) * up_n.
- * row_scale as in hymeta_moe_gemm. */
+ * gated != 0: W[e] is [2 N, K] (gate rows, then up rows) and out[slot, n] = silu(gate_n) * up_n (HYMETA_GLU_SILU), or
+ * g sigmoid(act_alpha g) (u + 1) with g = min(gate_n, act_limit), u = clamp(up_n, -act_limit, act_limit)
+ * (HYMETA_GLU_CLAMPED).  row_scale as in hymeta_moe_gemm. */
+enum hymeta_glu_mode { HYMETA_GLU_NONE = 0, HYMETA_GLU_SILU = 1, HYMETA_GLU_CLAMPED = 2 };
 typedef struct hymeta_moe_gemm_any_args {
   uint32_t struct_size;
   const void* x;               /* act_dtype rows of K */
@@ -1226,6 +1239,7 @@ typedef struct hymeta_moe_gemm_any_args {
   const float* row_scale;      /* or NULL */
   int32_t a_rows_div, max_rows, K, N, num_experts, gated, act_dtype;
   int64_t x_stride_m, out_stride_m, w_stride_e;
+  float act_limit, act_alpha;  /* gated == HYMETA_GLU_CLAMPED */
 } hymeta_moe_gemm_any_args;
 int hymeta_moe_gemm_any(const hymeta_moe_gemm_any_args* args, hymeta_stream_t stream);
 
@@ -1239,6 +1253,155 @@ typedef struct hymeta_moe_combine_any_args {
   int64_t y_stride_m, out_stride_m;
 } hymeta_moe_combine_any_args;
 int hymeta_moe_combine_any(const hymeta_moe_combine_any_args* args, hymeta_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Building blocks of post-norm designs with latent and linear attention.
+ * ---------------------------------------------------------------------- */
+
+/* Token shift of an fp32 stream: out[t] = x[t] + (x[t - 1] - x[t]) * mix, with x before a sequence's first token = 0.
+ * state fp32 [slots, width] holds every sequence's last row x between steps: read for the first row of a portion
+ * (context_lens > 0) and rewritten with the portion's last row in the same launch.  slot_idx < 0: no state. */
+typedef struct hymeta_token_shift_args {
+  uint32_t struct_size;
+  const float* x;              /* [num_tokens, width], row stride x_stride_t */
+  const float* mix;            /* [width] */
+  float* state;                /* [slots, width] */
+  void* out;                   /* act_dtype [num_tokens, width] contiguous */
+  const int32_t* query_start_loc;  /* [num_seqs + 1] */
+  const int32_t* context_lens;     /* [num_seqs] */
+  const int32_t* slot_idx;         /* [num_seqs] */
+  int32_t num_tokens, num_seqs, width, act_dtype;
+  int64_t x_stride_t;
+} hymeta_token_shift_args;
+int hymeta_token_shift(const hymeta_token_shift_args* args, hymeta_stream_t stream);
+
+/* Norm after the sum: z = alpha * x[t] (+ y[t]) (+ y2[t]), split into `groups` equal consecutive parts, each divided by
+ * its own sqrt(mean(part^2) + eps), times weight.  in_place != 0: written back to the fp32 stream x; out != NULL: (also)
+ * written to out, rounded to act_dtype (what the next sublayer's projections read; the model's last norm writes only
+ * this).  width % groups == 0. */
+typedef struct hymeta_add_group_norm_args {
+  uint32_t struct_size;
+  float* x;                    /* [num_tokens, width], row stride x_stride_t */
+  const void* y;               /* act_dtype [num_tokens, width], row stride y_stride_t, or NULL */
+  const void* y2;              /* act_dtype, row stride y2_stride_t, or NULL */
+  const float* weight;         /* [width] */
+  void* out;                   /* act_dtype [num_tokens, width] contiguous, or NULL */
+  int32_t num_tokens, width, groups, act_dtype, in_place;
+  float eps, alpha;
+  int64_t x_stride_t, y_stride_t, y2_stride_t;
+} hymeta_add_group_norm_args;
+int hymeta_add_group_norm(const hymeta_add_group_norm_args* args, hymeta_stream_t stream);
+
+/* Latent attention, the part between the down projections and the up projection of the queries.  proj holds, per
+ * token, the query latent (q_rank columns from q_col) and the key/value latent followed by the rotated key part shared
+ * by all heads (kv_rank + rot_dim columns from kv_col):
+ *   query latent  <- RMS norm with q_norm_weight, in place
+ *   cache row     <- (RMS norm of the key/value latent with kv_norm_weight, rotated key part)
+ * kv_cache: act_dtype [num_blocks, block_size, kv_rank + rot_dim].  The rotation turns the pair (2i, 2i + 1), i <
+ * rot_dims / 2 <= rot_dim / 2, by position * rot_freqs[i] (angles in double precision), cos and sin times rot_mag; the
+ * position of row t of sequence s is seq_lens[s] - (query_start_loc[s + 1] - t).  slot_mapping[t] < 0: no store. */
+typedef struct hymeta_latent_kv_prep_args {
+  uint32_t struct_size;
+  void* proj;                  /* act_dtype [num_tokens, ...], row stride proj_stride_t */
+  const float* q_norm_weight;  /* [q_rank] */
+  const float* kv_norm_weight; /* [kv_rank] */
+  const double* rot_freqs;     /* [rot_dims / 2] */
+  void* kv_cache;
+  const int64_t* slot_mapping; /* [num_tokens] */
+  const int32_t* query_start_loc;
+  const int32_t* seq_lens;
+  int32_t num_tokens, num_seqs, q_rank, kv_rank, rot_dim, rot_dims, q_col, kv_col, block_size, act_dtype;
+  float eps, rot_mag;
+  int64_t num_blocks, proj_stride_t;
+} hymeta_latent_kv_prep_args;
+int hymeta_latent_kv_prep(const hymeta_latent_kv_prep_args* args, hymeta_stream_t stream);
+
+/* The queries of a latent attention against the cached rows: out[t, h] = (q_abs[h, t] (kv_rank values: the unrotated
+ * query part carried through the keys' up projection), rotated q[t, h, dim:] (rot_dim values)). */
+typedef struct hymeta_latent_q_assemble_args {
+  uint32_t struct_size;
+  const void* q;               /* act_dtype [num_tokens, num_heads, dim + rot_dim], row stride q_stride_t */
+  const void* q_abs;           /* act_dtype [num_heads, num_tokens, kv_rank] contiguous */
+  void* out;                   /* act_dtype [num_tokens, num_heads, kv_rank + rot_dim] contiguous */
+  const double* rot_freqs;
+  const int32_t* query_start_loc;
+  const int32_t* seq_lens;
+  int32_t num_tokens, num_seqs, num_heads, dim, rot_dim, rot_dims, kv_rank, act_dtype;
+  float rot_mag;
+  int64_t q_stride_t;
+} hymeta_latent_q_assemble_args;
+int hymeta_latent_q_assemble(const hymeta_latent_q_assemble_args* args, hymeta_stream_t stream);
+
+/* Linear attention with a constant decay per head over a step's rows:
+ *   q, k, v = silu of the columns [0, H D), [H D, 2 H D), [2 H D, 2 H D + H Dv) of qkv
+ *   S <- decay[h] S + k v^T,   out = S^T q        (S fp32 [head_dim, v_dim] per sequence and head)
+ * state fp32 [slots, H, head_dim, v_dim] is read where context_lens > 0 (else the state starts at zero) and written.
+ * Portions of at least HYMETA_LIGHTNING_CHUNK rows of bf16 activations with head_dim and v_dim multiples of 32 up to 128
+ * run in chunks on the matrix cores; everything else token by token. */
+#define HYMETA_LIGHTNING_CHUNK 64
+typedef struct hymeta_lightning_attention_args {
+  uint32_t struct_size;
+  const void* qkv;             /* act_dtype [num_tokens, 2 H D + H Dv], row stride qkv_stride_t */
+  float* state;
+  const float* decay;          /* [num_heads] */
+  float* out;                  /* fp32 [num_tokens, H Dv] contiguous */
+  const int32_t* query_start_loc;
+  const int32_t* context_lens;
+  const int32_t* slot_idx;
+  int32_t num_tokens, num_seqs, num_heads, head_dim, v_dim, act_dtype, max_query_len;
+  int64_t qkv_stride_t;
+} hymeta_lightning_attention_args;
+int hymeta_lightning_attention(const hymeta_lightning_attention_args* args, hymeta_stream_t stream);
+
+/* out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * weight * sigmoid(gate[t]): the output norm and gate of a linear attention. */
+typedef struct hymeta_gated_rms_norm_args {
+  uint32_t struct_size;
+  const float* x;              /* fp32 [num_tokens, width] contiguous */
+  const void* gate;            /* act_dtype [num_tokens, width], row stride gate_stride_t */
+  const float* weight;         /* [width] */
+  void* out;                   /* act_dtype [num_tokens, width] contiguous */
+  int32_t num_tokens, width, act_dtype;
+  float eps;
+  int64_t gate_stride_t;
+} hymeta_gated_rms_norm_args;
+int hymeta_gated_rms_norm(const hymeta_gated_rms_norm_args* args, hymeta_stream_t stream);
+
+/* Elementwise activations between two projections, act_dtype in and out, fp32 inside:
+ *   HYMETA_ACT_CLAMPED_GLU  x [rows, 2 n] (gate columns, then up columns): g = min(gate, limit), u = clamp(up, -limit,
+ *                           limit), out = g sigmoid(alpha g) (u + 1)
+ *   HYMETA_ACT_XIELU        x [rows, n]: z > 0: a_pos z^2 + z / 2;  z <= 0: a_neg (exp(z) - 1 - z) + z / 2
+ *   HYMETA_ACT_SIGMOID_MUL  x [rows, n], gate [rows, n]: out = x * sigmoid(gate)
+ * num_rows_dev: optional device count of the rows in use; NULL: num_rows. */
+enum hymeta_act_kind { HYMETA_ACT_CLAMPED_GLU = 0, HYMETA_ACT_XIELU = 1, HYMETA_ACT_SIGMOID_MUL = 2 };
+typedef struct hymeta_activation_args {
+  uint32_t struct_size;
+  const void* x;               /* [rows, n or 2 n], row stride x_stride */
+  const void* gate;            /* HYMETA_ACT_SIGMOID_MUL: [rows, n], row stride gate_stride */
+  void* out;                   /* [rows, n], row stride out_stride */
+  const int32_t* num_rows_dev;
+  int32_t kind, num_rows, n, act_dtype;
+  float p0, p1;                /* CLAMPED_GLU: limit, alpha;  XIELU: a_pos, a_neg */
+  int64_t x_stride, gate_stride, out_stride;
+} hymeta_activation_args;
+int hymeta_activation(const hymeta_activation_args* args, hymeta_stream_t stream);
+
+/* Router of a mixture of experts with sigmoid scores: logits = x router_weight^T in fp32, s = sigmoid(logits), the top_k
+ * largest s are chosen (the lower expert on a tie), their weights are s / (sum of the chosen s + 1e-20) * scale.
+ * Writes what hymeta_moe_route writes.  num_experts <= HYMETA_MOE_TABLE_MAX_EXPERTS. */
+typedef struct hymeta_moe_route_sigmoid_args {
+  uint32_t struct_size;
+  const void* x;               /* act_dtype [num_tokens, hidden], row stride x_stride_t */
+  const float* router_weight;  /* [num_experts, hidden] contiguous */
+  int32_t* topk_ids;           /* out [num_tokens, top_k] */
+  float* topk_weights;         /* out [num_tokens, top_k] */
+  int32_t* expert_offsets;     /* out [num_experts + 1] */
+  int32_t* sorted_pair;        /* out [num_tokens * top_k] */
+  int32_t* pair_pos;           /* out [num_tokens * top_k] */
+  int32_t num_tokens, num_experts, top_k, hidden, act_dtype;
+  float scale;
+  int64_t x_stride_t;
+} hymeta_moe_route_sigmoid_args;
+int hymeta_moe_route_sigmoid(const hymeta_moe_route_sigmoid_args* args, hymeta_stream_t stream);
 
 #ifdef __cplusplus
 }

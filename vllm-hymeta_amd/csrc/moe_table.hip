@@ -130,7 +130,12 @@ __global__ __launch_bounds__(256) void moe_gemm_any_kernel(hymeta_moe_gemm_any_a
       float v = acc[r][c];
       if (Gated) {
         const float gte = A::round(v), up = A::round(acc2[r][c]);   // the two projections' outputs as a GEMM would store them
-        v = gte * sigmoid_exact(gte) * up;
+        if (a.gated == HYMETA_GLU_CLAMPED) {
+          const float gc = fminf(gte, a.act_limit), uc = fminf(fmaxf(up, -a.act_limit), a.act_limit);
+          v = gc * sigmoid_exact(a.act_alpha * gc) * (uc + 1.f);
+        } else {
+          v = gte * sigmoid_exact(gte) * up;
+        }
       }
       A::st(orow + n, v * sc);
     }
@@ -175,6 +180,7 @@ extern "C" int hymeta_moe_gemm_any(const hymeta_moe_gemm_any_args* args, hymeta_
   const hymeta_moe_gemm_any_args& a = *args;
   if (a.max_rows < 0 || a.K <= 0 || a.N <= 0 || a.num_experts <= 0) return HYMETA_ERR_INVALID_ARG;
   if (!act_dtype_ok(a.act_dtype)) return HYMETA_ERR_UNSUPPORTED;
+  if (a.gated != HYMETA_GLU_NONE && a.gated != HYMETA_GLU_SILU && a.gated != HYMETA_GLU_CLAMPED) return HYMETA_ERR_UNSUPPORTED;
   if (a.max_rows == 0) return HYMETA_OK;
   if (!a.x || !a.weights || !a.out || !a.expert_offsets) return HYMETA_ERR_INVALID_ARG;
   if (a.a_rows != nullptr && a.a_rows_div <= 0) return HYMETA_ERR_INVALID_ARG;

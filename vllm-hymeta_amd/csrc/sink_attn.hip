@@ -10,8 +10,8 @@ namespace hymeta {
 
 namespace {
 
-constexpr int kMaxHeadDim = 512;
-constexpr int kMaxVChunks = 4;       // value size <= 256
+constexpr int kMaxHeadDim = 1024;
+constexpr int kMaxVChunks = 8;       // value size <= 512
 
 // grid = tokens; a wave per (token, head) task: query heads, then key heads, then value heads.
 template <typename A>
@@ -79,10 +79,14 @@ __global__ __launch_bounds__(64) void sink_attention_rows_kernel(hymeta_sink_att
   for (int d = lane; d < D; d += 64) s_q[d] = A::ld(q + d);
   const int32_t* bt = a.block_tables + static_cast<int64_t>(s) * a.block_table_stride;
   const elem* cache = static_cast<const elem*>(a.kv_cache);
-  const int64_t row_elems = static_cast<int64_t>(G) * (D + Dv);
+  // a head's part of a cache row: its key followed by its value, or a key whose first Dv elements are the value
+  const int head_elems = a.kv_layout == HYMETA_KV_VALUE_IN_KEY ? D : D + Dv;
+  const int v_off = a.kv_layout == HYMETA_KV_VALUE_IN_KEY ? 0 : D;
+  const int64_t row_elems = static_cast<int64_t>(G) * head_elems;
   const float ba = a.bias_mode ? a.bias_a[h] : 0.f, bb = a.bias_mode ? a.bias_b[h] : 0.f;
-  float m = a.sink ? 0.f : -INFINITY, l = a.sink ? 1.f : 0.f;
-  float acc[kMaxVChunks] = {0.f, 0.f, 0.f, 0.f};
+  // the sink: a key of score sink_logits[h] (0 without) that has no value
+  float m = a.sink ? (a.sink_logits ? a.sink_logits[h] : 0.f) : -INFINITY, l = a.sink ? 1.f : 0.f;
+  float acc[kMaxVChunks] = {};
   const int nvc = (Dv + 63) / 64;
   __syncthreads();
   for (int j0 = first; j0 <= pos; j0 += 64) {
@@ -92,7 +96,7 @@ __global__ __launch_bounds__(64) void sink_attention_rows_kernel(hymeta_sink_att
     int64_t roff = 0;
     if (valid) {
       const int64_t blk = bt[j / a.block_size];
-      roff = (blk * a.block_size + j % a.block_size) * row_elems + static_cast<int64_t>(g) * (D + Dv);
+      roff = (blk * a.block_size + j % a.block_size) * row_elems + static_cast<int64_t>(g) * head_elems;
       const elem* k = cache + roff;
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot = fmaf(s_q[d], A::ld(k + d), dot);
@@ -105,7 +109,7 @@ __global__ __launch_bounds__(64) void sink_attention_rows_kernel(hymeta_sink_att
     m = m_new;
     __syncthreads();
     s_p[lane] = p;
-    s_row[lane] = roff + D;
+    s_row[lane] = roff + v_off;
     __syncthreads();
     const int n = min(64, pos - j0 + 1);
 #pragma unroll
@@ -416,8 +420,8 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void sink_attention_prefill_mfm
     w.pos[rb] = ok ? ctx + r : -1;
     w.ba[rb] = a.bias_mode ? a.bias_a[h] : 0.f;
     w.bb[rb] = a.bias_mode ? a.bias_b[h] : 0.f;
-    w.m[rb] = a.sink ? 0.f : -INFINITY;
-    w.l[rb] = (a.sink && g4 == 0) ? 1.f : 0.f;        // the sink's exp(0 - 0), counted once per row
+    w.m[rb] = a.sink ? (a.sink_logits ? a.sink_logits[h] * 1.4426950408889634f : 0.f) : -INFINITY;
+    w.l[rb] = (a.sink && g4 == 0) ? 1.f : 0.f;        // the sink's exp(m - m), counted once per row
     load_q<D, DV, RB>(w, rb, ok ? static_cast<const uint16_t*>(a.q) + static_cast<int64_t>(row0 + r) * a.q_stride_t + static_cast<int64_t>(h) * D : nullptr);
 #pragma unroll
     for (int cb = 0; cb < DV / 16; ++cb) w.o[rb][cb] = f32x4v{0.f, 0.f, 0.f, 0.f};
@@ -544,9 +548,10 @@ __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymet
   const float* base = static_cast<const float*>(a.workspace) + (static_cast<size_t>(s) * a.num_kv_heads + g) * splits * stride +
                       r * partial_row_floats(DV);
   // (the partials' maxima are in the base-2 domain, as the waves kept them)
-  float m = a.sink ? 0.f : -INFINITY;
+  const float sink2 = a.sink_logits ? a.sink_logits[h] * 1.4426950408889634f : 0.f;
+  float m = a.sink ? sink2 : -INFINITY;
   for (int sp = 0; sp < splits; ++sp) m = fmaxf(m, base[sp * stride + DV]);
-  float l = a.sink ? __builtin_amdgcn_exp2f(0.f - m) : 0.f;
+  float l = a.sink ? __builtin_amdgcn_exp2f(sink2 - m) : 0.f;
   for (int sp = 0; sp < splits; ++sp) {
     const float ms = base[sp * stride + DV];
     if (ms != -INFINITY) l += base[sp * stride + DV + 1] * __builtin_amdgcn_exp2f(ms - m);
@@ -565,7 +570,8 @@ __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymet
 
 inline bool mfma_shape(const hymeta_sink_attention_args& a) {
   const bool dims = (a.head_dim == 64 || a.head_dim == 128) && (a.v_dim == 64 || a.v_dim == 128);
-  return a.act_dtype == HYMETA_BF16 && dims && a.num_heads / a.num_kv_heads <= kRowsPerWave && a.q_stride_t % 8 == 0 &&
+  return a.act_dtype == HYMETA_BF16 && dims && a.kv_layout == HYMETA_KV_KEY_THEN_VALUE && a.num_heads / a.num_kv_heads <= kRowsPerWave &&
+         a.q_stride_t % 8 == 0 &&
          (a.block_size & (a.block_size - 1)) == 0 &&
          (reinterpret_cast<uintptr_t>(a.q) | reinterpret_cast<uintptr_t>(a.kv_cache) | reinterpret_cast<uintptr_t>(a.out)) % 16 == 0;
 }
@@ -637,6 +643,8 @@ extern "C" int hymeta_sink_attention(const hymeta_sink_attention_args* args, hym
   if (!act_dtype_ok(a.act_dtype)) return HYMETA_ERR_UNSUPPORTED;
   if (a.head_dim > kMaxHeadDim || a.v_dim > 64 * kMaxVChunks) return HYMETA_ERR_UNSUPPORTED;
   if (a.bias_mode != HYMETA_BIAS_NONE && a.bias_mode != HYMETA_BIAS_LOG_DISTANCE) return HYMETA_ERR_UNSUPPORTED;
+  if (a.kv_layout != HYMETA_KV_KEY_THEN_VALUE && a.kv_layout != HYMETA_KV_VALUE_IN_KEY) return HYMETA_ERR_UNSUPPORTED;
+  if (a.kv_layout == HYMETA_KV_VALUE_IN_KEY && a.v_dim > a.head_dim) return HYMETA_ERR_INVALID_ARG;
   if (a.num_tokens == 0 || a.num_seqs == 0) return HYMETA_OK;
   if (!a.q || !a.kv_cache || !a.out || !a.block_tables || !a.query_start_loc || !a.seq_lens) return HYMETA_ERR_INVALID_ARG;
   if (a.bias_mode != HYMETA_BIAS_NONE && (!a.bias_a || !a.bias_b)) return HYMETA_ERR_INVALID_ARG;

@@ -26,9 +26,14 @@ GATE_70B_LOWER_BOUND = 3
 
 BIAS_NONE = 0
 BIAS_LOG_DISTANCE = 1
+KV_KEY_THEN_VALUE = 0
+KV_VALUE_IN_KEY = 1
+GLU_NONE, GLU_SILU, GLU_CLAMPED = 0, 1, 2
+ACT_CLAMPED_GLU, ACT_XIELU, ACT_SIGMOID_MUL = 0, 1, 2
+LIGHTNING_CHUNK = 64
 CONV_MAX_TAPS = 8
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 ERR_SCRATCH_LIMIT = -5
 GEMM_TICKET_BYTES = 16384
 STATIC_SCRATCH_BYTES = 16 << 20
@@ -351,6 +356,7 @@ class SinkAttentionArgs(_Args):
         ("bias_mode", _i32), ("sink", _i32), ("window_left", _i32), ("max_query_len", _i32), ("max_seq_len", _i32),
         ("scale", _f32),
         ("num_blocks", _i64), ("q_stride_t", _i64), ("block_table_stride", _i64),
+        ("sink_logits", _ptr), ("kv_layout", _i32),
     ]
 
 
@@ -371,6 +377,7 @@ class MoeGemmAnyArgs(_Args):
         ("a_rows_div", _i32), ("max_rows", _i32), ("K", _i32), ("N", _i32), ("num_experts", _i32), ("gated", _i32),
         ("act_dtype", _i32),
         ("x_stride_m", _i64), ("out_stride_m", _i64), ("w_stride_e", _i64),
+        ("act_limit", _f32), ("act_alpha", _f32),
     ]
 
 
@@ -380,6 +387,91 @@ class MoeCombineAnyArgs(_Args):
         ("y", _ptr), ("out", _ptr), ("pair_pos", _ptr),
         ("num_tokens", _i32), ("width", _i32), ("top_k", _i32), ("act_dtype", _i32),
         ("y_stride_m", _i64), ("out_stride_m", _i64),
+    ]
+
+
+class TokenShiftArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("x", _ptr), ("mix", _ptr), ("state", _ptr), ("out", _ptr),
+        ("query_start_loc", _ptr), ("context_lens", _ptr), ("slot_idx", _ptr),
+        ("num_tokens", _i32), ("num_seqs", _i32), ("width", _i32), ("act_dtype", _i32),
+        ("x_stride_t", _i64),
+    ]
+
+
+class AddGroupNormArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("x", _ptr), ("y", _ptr), ("y2", _ptr), ("weight", _ptr), ("out", _ptr),
+        ("num_tokens", _i32), ("width", _i32), ("groups", _i32), ("act_dtype", _i32), ("in_place", _i32),
+        ("eps", _f32), ("alpha", _f32),
+        ("x_stride_t", _i64), ("y_stride_t", _i64), ("y2_stride_t", _i64),
+    ]
+
+
+class LatentKvPrepArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("proj", _ptr), ("q_norm_weight", _ptr), ("kv_norm_weight", _ptr), ("rot_freqs", _ptr), ("kv_cache", _ptr),
+        ("slot_mapping", _ptr), ("query_start_loc", _ptr), ("seq_lens", _ptr),
+        ("num_tokens", _i32), ("num_seqs", _i32), ("q_rank", _i32), ("kv_rank", _i32), ("rot_dim", _i32), ("rot_dims", _i32),
+        ("q_col", _i32), ("kv_col", _i32), ("block_size", _i32), ("act_dtype", _i32),
+        ("eps", _f32), ("rot_mag", _f32),
+        ("num_blocks", _i64), ("proj_stride_t", _i64),
+    ]
+
+
+class LatentQAssembleArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("q", _ptr), ("q_abs", _ptr), ("out", _ptr), ("rot_freqs", _ptr), ("query_start_loc", _ptr), ("seq_lens", _ptr),
+        ("num_tokens", _i32), ("num_seqs", _i32), ("num_heads", _i32), ("dim", _i32), ("rot_dim", _i32), ("rot_dims", _i32),
+        ("kv_rank", _i32), ("act_dtype", _i32),
+        ("rot_mag", _f32),
+        ("q_stride_t", _i64),
+    ]
+
+
+class LightningAttentionArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("qkv", _ptr), ("state", _ptr), ("decay", _ptr), ("out", _ptr),
+        ("query_start_loc", _ptr), ("context_lens", _ptr), ("slot_idx", _ptr),
+        ("num_tokens", _i32), ("num_seqs", _i32), ("num_heads", _i32), ("head_dim", _i32), ("v_dim", _i32), ("act_dtype", _i32),
+        ("max_query_len", _i32),
+        ("qkv_stride_t", _i64),
+    ]
+
+
+class GatedRmsNormArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("x", _ptr), ("gate", _ptr), ("weight", _ptr), ("out", _ptr),
+        ("num_tokens", _i32), ("width", _i32), ("act_dtype", _i32),
+        ("eps", _f32),
+        ("gate_stride_t", _i64),
+    ]
+
+
+class ActivationArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("x", _ptr), ("gate", _ptr), ("out", _ptr), ("num_rows_dev", _ptr),
+        ("kind", _i32), ("num_rows", _i32), ("n", _i32), ("act_dtype", _i32),
+        ("p0", _f32), ("p1", _f32),
+        ("x_stride", _i64), ("gate_stride", _i64), ("out_stride", _i64),
+    ]
+
+
+class MoeRouteSigmoidArgs(_Args):
+    _fields_ = [
+        _SIZE,
+        ("x", _ptr), ("router_weight", _ptr), ("topk_ids", _ptr), ("topk_weights", _ptr), ("expert_offsets", _ptr),
+        ("sorted_pair", _ptr), ("pair_pos", _ptr),
+        ("num_tokens", _i32), ("num_experts", _i32), ("top_k", _i32), ("hidden", _i32), ("act_dtype", _i32),
+        ("scale", _f32),
+        ("x_stride_t", _i64),
     ]
 
 
@@ -461,6 +553,14 @@ _SIGNATURES = {
     "hymeta_moe_route_table": (C.c_int, [C.POINTER(MoeRouteTableArgs), _ptr]),
     "hymeta_moe_gemm_any": (C.c_int, [C.POINTER(MoeGemmAnyArgs), _ptr]),
     "hymeta_moe_combine_any": (C.c_int, [C.POINTER(MoeCombineAnyArgs), _ptr]),
+    "hymeta_token_shift": (C.c_int, [C.POINTER(TokenShiftArgs), _ptr]),
+    "hymeta_add_group_norm": (C.c_int, [C.POINTER(AddGroupNormArgs), _ptr]),
+    "hymeta_latent_kv_prep": (C.c_int, [C.POINTER(LatentKvPrepArgs), _ptr]),
+    "hymeta_latent_q_assemble": (C.c_int, [C.POINTER(LatentQAssembleArgs), _ptr]),
+    "hymeta_lightning_attention": (C.c_int, [C.POINTER(LightningAttentionArgs), _ptr]),
+    "hymeta_gated_rms_norm": (C.c_int, [C.POINTER(GatedRmsNormArgs), _ptr]),
+    "hymeta_activation": (C.c_int, [C.POINTER(ActivationArgs), _ptr]),
+    "hymeta_moe_route_sigmoid": (C.c_int, [C.POINTER(MoeRouteSigmoidArgs), _ptr]),
 }
 
 STRUCTS = {
@@ -491,6 +591,14 @@ STRUCTS = {
     "hymeta_moe_route_table_args": MoeRouteTableArgs,
     "hymeta_moe_gemm_any_args": MoeGemmAnyArgs,
     "hymeta_moe_combine_any_args": MoeCombineAnyArgs,
+    "hymeta_token_shift_args": TokenShiftArgs,
+    "hymeta_add_group_norm_args": AddGroupNormArgs,
+    "hymeta_latent_kv_prep_args": LatentKvPrepArgs,
+    "hymeta_latent_q_assemble_args": LatentQAssembleArgs,
+    "hymeta_lightning_attention_args": LightningAttentionArgs,
+    "hymeta_gated_rms_norm_args": GatedRmsNormArgs,
+    "hymeta_activation_args": ActivationArgs,
+    "hymeta_moe_route_sigmoid_args": MoeRouteSigmoidArgs,
 }
 
 

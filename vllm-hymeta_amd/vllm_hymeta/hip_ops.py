@@ -1599,15 +1599,20 @@ def qk_norm_cache_(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
 def sink_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_tables: torch.Tensor, query_start_loc: torch.Tensor,
                    seq_lens: torch.Tensor, num_kv_heads: int, head_dim: int, v_dim: int, scale: float,
                    max_query_len: int, max_seq_len: int, bias_a: Optional[torch.Tensor] = None,
-                   bias_b: Optional[torch.Tensor] = None, sink: bool = True, window_left: int = -1) -> torch.Tensor:
+                   bias_b: Optional[torch.Tensor] = None, sink: bool = True, window_left: int = -1,
+                   sink_logits: Optional[torch.Tensor] = None, value_in_key: bool = False) -> torch.Tensor:
     """Causal attention of the rows ``q [T, H, D]`` over their sequences' paged keys (this step's included):
-    ``softmax`` over ``scale q.k - bias_a[h] ln(1 + bias_b[h] (i - j))`` with, for ``sink``, one added to the denominator.
-    Returns ``[T, H, Dv]``."""
-    _dev(q, kv_cache, block_tables, query_start_loc, seq_lens, bias_a, bias_b)
+    ``softmax`` over ``scale q.k - bias_a[h] ln(1 + bias_b[h] (i - j))`` with, for ``sink``, ``exp(sink_logits[h])`` (one
+    without ``sink_logits``) added to the denominator.  ``value_in_key``: a cache row holds ``D`` elements per key/value
+    head, the first ``Dv`` of which are also the value (a latent that keys and values share).  Returns ``[T, H, Dv]``."""
+    _dev(q, kv_cache, block_tables, query_start_loc, seq_lens, bias_a, bias_b, sink_logits)
     _require(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == head_dim and q.shape[2] == head_dim, "q must be [T, H, D] with contiguous heads")
     T, H, _ = q.shape
+    row = head_dim if value_in_key else head_dim + v_dim
+    _require(not value_in_key or v_dim <= head_dim, "a value inside its key cannot be longer than the key")
     _require(kv_cache.dtype == q.dtype and kv_cache.is_contiguous() and kv_cache.dim() == 4
-             and kv_cache.shape[2:] == (num_kv_heads, head_dim + v_dim), "kv_cache must be contiguous [blocks, block_size, G, D + Dv]")
+             and kv_cache.shape[2:] == (num_kv_heads, row), f"kv_cache must be contiguous [blocks, block_size, G, {row}]")
+    _f32vec(sink_logits, H, "sink_logits")
     S = query_start_loc.numel() - 1
     _i32vec(query_start_loc, S + 1, "query_start_loc")
     _i32vec(seq_lens, S, "seq_lens")
@@ -1629,6 +1634,7 @@ def sink_attention(q: torch.Tensor, kv_cache: torch.Tensor, block_tables: torch.
     a.block_size, a.act_dtype, a.num_blocks = kv_cache.shape[1], _act(q), kv_cache.shape[0]
     a.bias_mode = _C.BIAS_NONE if bias_a is None else _C.BIAS_LOG_DISTANCE
     a.sink, a.window_left, a.max_query_len, a.max_seq_len, a.scale = int(bool(sink)), window_left, max_query_len, max_seq_len, scale
+    a.sink_logits, a.kv_layout = _p(sink_logits), (_C.KV_VALUE_IN_KEY if value_in_key else _C.KV_KEY_THEN_VALUE)
     a.q_stride_t, a.block_table_stride = q.stride(0), block_tables.stride(0)
     _C.check(lib.hymeta_sink_attention(C.byref(a), _stream(q)), "hymeta_sink_attention")
     return out
@@ -1713,6 +1719,272 @@ def moe_table_forward(x: torch.Tensor, token_ids: torch.Tensor, table: torch.Ten
     c = _C.MoeCombineAnyArgs()
     c.y, c.out, c.pair_pos = _p(y), _p(out), _p(pair_pos)
     c.num_tokens, c.width, c.top_k, c.act_dtype = T, H, top, act
+    c.y_stride_m, c.out_stride_m = y.stride(0), out.stride(0)
+    _C.check(lib.hymeta_moe_combine_any(C.byref(c), st), "hymeta_moe_combine_any")
+    return out
+
+
+# ---------------------------------------------------------------------------
+# Building blocks of post-norm designs with latent and linear attention.
+# ---------------------------------------------------------------------------
+def token_shift(x: torch.Tensor, mix: torch.Tensor, state: Optional[torch.Tensor], out_dtype: torch.dtype,
+                query_start_loc: torch.Tensor, context_lens: torch.Tensor, slot_idx: Optional[torch.Tensor]) -> torch.Tensor:
+    """``x[t] + (x[t - 1] - x[t]) * mix`` over each sequence's rows of the fp32 stream ``x [T, W]`` (zeros before a
+    sequence's first token); ``state`` fp32 ``[slots, W]`` carries a sequence's last row between steps, in place."""
+    _dev(x, mix, state, query_start_loc, context_lens, slot_idx)
+    _require(x.dim() == 2 and x.dtype == torch.float32 and x.stride(1) == 1, "x must be row-contiguous fp32 [T, W]")
+    T, W = x.shape
+    _f32vec(mix, W, "mix")
+    _require(out_dtype in _DT, "out_dtype must be bf16 or fp32")
+    S = query_start_loc.numel() - 1
+    _i32vec(query_start_loc, S + 1, "query_start_loc")
+    _i32vec(context_lens, S, "context_lens")
+    out = torch.empty(T, W, dtype=out_dtype, device=x.device)
+    a = _C.TokenShiftArgs()
+    a.x, a.mix, a.out, a.query_start_loc, a.context_lens = _p(x), _p(mix), _p(out), _p(query_start_loc), _p(context_lens)
+    if state is not None:
+        _require(slot_idx is not None, "state needs slot_idx")
+        _i32vec(slot_idx, S, "slot_idx")
+        _require(state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 2 and state.shape[1] == W,
+                 "state must be contiguous fp32 [slots, W]")
+        a.state, a.slot_idx = _p(state), _p(slot_idx)
+    a.num_tokens, a.num_seqs, a.width, a.act_dtype, a.x_stride_t = T, S, W, _DT[out_dtype], x.stride(0)
+    _C.check(_C.load().hymeta_token_shift(C.byref(a), _stream(x)), "hymeta_token_shift")
+    return out
+
+
+def add_group_norm(x: torch.Tensor, y: Optional[torch.Tensor], weight: torch.Tensor, groups: int, eps: float, alpha: float = 1.0,
+                   y2: Optional[torch.Tensor] = None, in_place: bool = True, out_dtype: Optional[torch.dtype] = None):
+    """``norm(alpha x + y (+ y2))`` with the RMS taken over each of ``groups`` equal consecutive parts of a row, times
+    ``weight``.  ``in_place``: written back into the fp32 stream ``x [T, W]``; ``out_dtype``: (also) returned as a new tensor
+    of that type (the rounded copy the next projections read).  Returns that tensor, or ``x``."""
+    _dev(x, y, y2, weight)
+    _require(x.dim() == 2 and x.dtype == torch.float32 and x.stride(1) == 1, "x must be row-contiguous fp32 [T, W]")
+    T, W = x.shape
+    _require(groups >= 1 and W % groups == 0, "the width must split into equal groups")
+    _require(in_place or out_dtype is not None, "the result must go somewhere")
+    _f32vec(weight, W, "weight")
+    act = None
+    for t, name in ((y, "y"), (y2, "y2")):
+        if t is not None:
+            _require(t.shape == (T, W) and t.stride(1) == 1 and t.dtype in _DT, f"{name} must be row-contiguous [T, W], bf16 or fp32")
+            _require(act is None or act == t.dtype, "y and y2 must share a type")
+            act = t.dtype
+    if out_dtype is not None:
+        _require(out_dtype in _DT and (act is None or act == out_dtype), "out_dtype must be the activations' type")
+        act = out_dtype
+    out = None if out_dtype is None else torch.empty(T, W, dtype=out_dtype, device=x.device)
+    a = _C.AddGroupNormArgs()
+    a.x, a.y, a.y2, a.weight, a.out = _p(x), _p(y), _p(y2), _p(weight), _p(out)
+    a.num_tokens, a.width, a.groups, a.act_dtype, a.in_place = T, W, groups, _DT[act or torch.float32], int(in_place)
+    a.eps, a.alpha, a.x_stride_t = eps, alpha, x.stride(0)
+    a.y_stride_t, a.y2_stride_t = (0 if y is None else y.stride(0)), (0 if y2 is None else y2.stride(0))
+    _C.check(_C.load().hymeta_add_group_norm(C.byref(a), _stream(x)), "hymeta_add_group_norm")
+    return x if out is None else out
+
+
+def latent_kv_prep_(proj: torch.Tensor, q_col: int, q_rank: int, kv_col: int, kv_rank: int, rot_dim: int, rot_dims: int,
+                    q_norm_weight: torch.Tensor, kv_norm_weight: torch.Tensor, eps: float, rot_freqs: torch.Tensor, rot_mag: float,
+                    kv_cache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor], query_start_loc: torch.Tensor,
+                    seq_lens: torch.Tensor) -> None:
+    """On the rows ``proj [T, ...]`` of the fused down projections: RMS norm of the query latent (columns ``q_col ..``) in
+    place; RMS norm of the key/value latent (columns ``kv_col ..``) and rotation of the ``rot_dim`` columns behind it,
+    both written to ``kv_cache [blocks, block_size, 1, kv_rank + rot_dim]`` at ``slot_mapping``."""
+    _dev(proj, q_norm_weight, kv_norm_weight, rot_freqs, kv_cache, slot_mapping, query_start_loc, seq_lens)
+    _require(proj.dim() == 2 and proj.stride(1) == 1, "proj must be row-contiguous")
+    T = proj.shape[0]
+    _require(q_col + q_rank <= proj.shape[1] and kv_col + kv_rank + rot_dim <= proj.shape[1], "the latents' columns must lie inside proj")
+    _f32vec(q_norm_weight, q_rank, "q_norm_weight")
+    _f32vec(kv_norm_weight, kv_rank, "kv_norm_weight")
+    _require(rot_freqs.dtype == torch.float64 and rot_freqs.is_contiguous() and rot_freqs.numel() * 2 >= rot_dims, "rot_freqs must be float64 [rot_dims / 2]")
+    S = query_start_loc.numel() - 1
+    _i32vec(query_start_loc, S + 1, "query_start_loc")
+    _i32vec(seq_lens, S, "seq_lens")
+    a = _C.LatentKvPrepArgs()
+    a.proj, a.q_norm_weight, a.kv_norm_weight, a.rot_freqs = _p(proj), _p(q_norm_weight), _p(kv_norm_weight), _p(rot_freqs)
+    a.query_start_loc, a.seq_lens = _p(query_start_loc), _p(seq_lens)
+    a.num_tokens, a.num_seqs, a.q_rank, a.kv_rank, a.rot_dim, a.rot_dims, a.q_col, a.kv_col = T, S, q_rank, kv_rank, rot_dim, rot_dims, q_col, kv_col
+    a.block_size, a.act_dtype, a.eps, a.rot_mag, a.proj_stride_t = 1, _act(proj), eps, rot_mag, proj.stride(0)
+    if kv_cache is not None and kv_cache.numel() > 0 and slot_mapping is not None:
+        _require(kv_cache.dtype == proj.dtype and kv_cache.is_contiguous() and kv_cache.dim() == 4 and kv_cache.shape[2:] == (1, kv_rank + rot_dim),
+                 "kv_cache must be contiguous [blocks, block_size, 1, kv_rank + rot_dim]")
+        _require(slot_mapping.dtype == torch.int64 and slot_mapping.is_contiguous() and slot_mapping.numel() == T, "slot_mapping must be int64 [T]")
+        a.kv_cache, a.slot_mapping, a.num_blocks, a.block_size = _p(kv_cache), _p(slot_mapping), kv_cache.shape[0], kv_cache.shape[1]
+    _C.check(_C.load().hymeta_latent_kv_prep(C.byref(a), _stream(proj)), "hymeta_latent_kv_prep")
+
+
+def latent_q_assemble(q: torch.Tensor, q_abs: torch.Tensor, dim: int, rot_dim: int, rot_dims: int, rot_freqs: torch.Tensor,
+                      rot_mag: float, query_start_loc: torch.Tensor, seq_lens: torch.Tensor) -> torch.Tensor:
+    """``q [T, H, dim + rot_dim]`` and ``q_abs [H, T, C]`` -> ``[T, H, C + rot_dim]``: the absorbed part followed by the
+    rotated part of every head's query."""
+    _dev(q, q_abs, rot_freqs, query_start_loc, seq_lens)
+    _require(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == dim + rot_dim and q.shape[2] == dim + rot_dim, "q must be [T, H, dim + rot_dim]")
+    T, H, _ = q.shape
+    _require(q_abs.dim() == 3 and q_abs.is_contiguous() and q_abs.shape[:2] == (H, T) and q_abs.dtype == q.dtype, "q_abs must be contiguous [H, T, C]")
+    Ck = q_abs.shape[2]
+    _require(rot_freqs.dtype == torch.float64 and rot_freqs.is_contiguous() and rot_freqs.numel() * 2 >= rot_dims, "rot_freqs must be float64 [rot_dims / 2]")
+    S = query_start_loc.numel() - 1
+    _i32vec(query_start_loc, S + 1, "query_start_loc")
+    _i32vec(seq_lens, S, "seq_lens")
+    out = torch.empty(T, H, Ck + rot_dim, dtype=q.dtype, device=q.device)
+    a = _C.LatentQAssembleArgs()
+    a.q, a.q_abs, a.out, a.rot_freqs, a.query_start_loc, a.seq_lens = _p(q), _p(q_abs), _p(out), _p(rot_freqs), _p(query_start_loc), _p(seq_lens)
+    a.num_tokens, a.num_seqs, a.num_heads, a.dim, a.rot_dim, a.rot_dims, a.kv_rank, a.act_dtype = T, S, H, dim, rot_dim, rot_dims, Ck, _act(q)
+    a.rot_mag, a.q_stride_t = rot_mag, q.stride(0)
+    _C.check(_C.load().hymeta_latent_q_assemble(C.byref(a), _stream(q)), "hymeta_latent_q_assemble")
+    return out
+
+
+def lightning_attention(qkv: torch.Tensor, state: torch.Tensor, decay: torch.Tensor, num_heads: int, head_dim: int, v_dim: int,
+                        query_start_loc: torch.Tensor, context_lens: torch.Tensor, slot_idx: torch.Tensor, max_query_len: int) -> torch.Tensor:
+    """Linear attention with a decay per head over a step's rows: ``qkv [T, 2 H D + H Dv]`` (before their silu), ``state``
+    fp32 ``[slots, H, D, Dv]`` read where ``context_lens > 0`` and written.  Returns fp32 ``[T, H Dv]``."""
+    _dev(qkv, state, decay, query_start_loc, context_lens, slot_idx)
+    H, D, Dv = num_heads, head_dim, v_dim
+    _require(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= H * (2 * D + Dv), "qkv must be row-contiguous [T, 2 H D + H Dv]")
+    _require(state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 4 and state.shape[1:] == (H, D, Dv),
+             "state must be contiguous fp32 [slots, H, D, Dv]")
+    _f32vec(decay, H, "decay")
+    T = qkv.shape[0]
+    S = query_start_loc.numel() - 1
+    _i32vec(query_start_loc, S + 1, "query_start_loc")
+    _i32vec(context_lens, S, "context_lens")
+    _i32vec(slot_idx, S, "slot_idx")
+    out = torch.empty(T, H * Dv, dtype=torch.float32, device=qkv.device)
+    a = _C.LightningAttentionArgs()
+    a.qkv, a.state, a.decay, a.out = _p(qkv), _p(state), _p(decay), _p(out)
+    a.query_start_loc, a.context_lens, a.slot_idx = _p(query_start_loc), _p(context_lens), _p(slot_idx)
+    a.num_tokens, a.num_seqs, a.num_heads, a.head_dim, a.v_dim, a.act_dtype, a.max_query_len = T, S, H, D, Dv, _act(qkv), max_query_len
+    a.qkv_stride_t = qkv.stride(0)
+    _C.check(_C.load().hymeta_lightning_attention(C.byref(a), _stream(qkv)), "hymeta_lightning_attention")
+    return out
+
+
+def gated_rms_norm(x: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """``rmsnorm(x) * weight * sigmoid(gate)``: fp32 rows ``x [T, W]``, ``gate [T, W]`` in the activations' type, which
+    is also the result's."""
+    _dev(x, gate, weight)
+    _require(x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous(), "x must be contiguous fp32 [T, W]")
+    T, W = x.shape
+    _require(gate.shape == (T, W) and gate.stride(1) == 1, "gate must be row-contiguous [T, W]")
+    _f32vec(weight, W, "weight")
+    out = torch.empty(T, W, dtype=gate.dtype, device=x.device)
+    a = _C.GatedRmsNormArgs()
+    a.x, a.gate, a.weight, a.out = _p(x), _p(gate), _p(weight), _p(out)
+    a.num_tokens, a.width, a.act_dtype, a.eps, a.gate_stride_t = T, W, _act(gate), eps, gate.stride(0)
+    _C.check(_C.load().hymeta_gated_rms_norm(C.byref(a), _stream(x)), "hymeta_gated_rms_norm")
+    return out
+
+
+def _activation(kind: int, x: torch.Tensor, n: int, p0: float, p1: float, gate: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None, num_rows_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(x, gate, out, num_rows_dev)
+    _require(x.dim() == 2 and x.stride(1) == 1, "x must be row-contiguous")
+    rows = x.shape[0]
+    if out is None:
+        out = torch.empty(rows, n, dtype=x.dtype, device=x.device)
+    _require(out.shape == (rows, n) and out.stride(1) == 1 and out.dtype == x.dtype, "out must be row-contiguous [rows, n] of x's type")
+    a = _C.ActivationArgs()
+    a.x, a.gate, a.out, a.num_rows_dev = _p(x), _p(gate), _p(out), _p(num_rows_dev)
+    a.kind, a.num_rows, a.n, a.act_dtype, a.p0, a.p1 = kind, rows, n, _act(x), p0, p1
+    a.x_stride, a.gate_stride, a.out_stride = x.stride(0), (0 if gate is None else gate.stride(0)), out.stride(0)
+    _C.check(_C.load().hymeta_activation(C.byref(a), _stream(x)), "hymeta_activation")
+    return out
+
+
+def clamped_glu(x: torch.Tensor, limit: float, alpha: float = 1.702, out: Optional[torch.Tensor] = None,
+                num_rows_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x [rows, 2 n]`` (gate columns, then up columns) -> ``g sigmoid(alpha g) (u + 1)`` with ``g = min(gate, limit)``,
+    ``u = clamp(up, -limit, limit)``."""
+    _require(x.shape[1] % 2 == 0, "x must hold the gate and the up columns")
+    return _activation(_C.ACT_CLAMPED_GLU, x, x.shape[1] // 2, limit, alpha, out=out, num_rows_dev=num_rows_dev)
+
+
+def xielu(x: torch.Tensor, a_pos: float, a_neg: float) -> torch.Tensor:
+    """``z > 0: a_pos z^2 + z / 2``; ``z <= 0: a_neg (exp(z) - 1 - z) + z / 2``."""
+    return _activation(_C.ACT_XIELU, x, x.shape[1], a_pos, a_neg)
+
+
+def sigmoid_gate_mul(x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """``x * sigmoid(gate)``, both ``[rows, n]``."""
+    _require(gate.shape == x.shape and gate.stride(1) == 1 and gate.dtype == x.dtype, "gate must be row-contiguous, of x's shape and type")
+    return _activation(_C.ACT_SIGMOID_MUL, x, x.shape[1], 0.0, 0.0, gate=gate)
+
+
+def moe_sigmoid_forward(x: torch.Tensor, router_weight: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, top_k: int,
+                        route_scale: float, limit: float, alpha: float = 1.702) -> torch.Tensor:
+    """Experts chosen by the ``top_k`` largest ``sigmoid(x router_weight^T)`` (fp32), weighing their scores over the
+    chosen's sum times ``route_scale``; every expert is a clamped gated unit (``clamped_glu``) between ``w13 [E, 2I, H]``
+    (gate rows, then up rows) and ``w2 [E, H, I]``, all bf16 or all fp32.  bf16 experts in the MFMA tiles' shapes run the
+    routed block's grouped GEMMs, everything else the generic grouped GEMM with the activation in its epilogue."""
+    _dev(x, router_weight, w13, w2)
+    T, H = x.shape
+    E, two_i, _ = w13.shape
+    inter = two_i // 2
+    _require(x.dtype in _DT and x.stride(1) == 1 and w13.dtype == x.dtype and w2.dtype == x.dtype, "x, w13 and w2 must share bf16 or fp32")
+    _require(w13.is_contiguous() and w13.shape == (E, 2 * inter, H) and w2.is_contiguous() and w2.shape == (E, H, inter),
+             "w13 must be contiguous [E, 2I, H] and w2 [E, H, I]")
+    _require(router_weight.dtype == torch.float32 and router_weight.is_contiguous() and router_weight.shape == (E, H),
+             "router_weight must be contiguous fp32 [E, H]")
+    dev = x.device
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    if T == 0:
+        return out
+    P = T * top_k
+    ids = torch.empty(T, top_k, dtype=torch.int32, device=dev)
+    wts = torch.empty(T, top_k, dtype=torch.float32, device=dev)
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    sorted_pair = torch.empty(P, dtype=torch.int32, device=dev)
+    pair_pos = torch.empty(P, dtype=torch.int32, device=dev)
+    lib, st = _C.load(), _stream(x)
+    r = _C.MoeRouteSigmoidArgs()
+    r.x, r.router_weight, r.topk_ids, r.topk_weights = _p(x), _p(router_weight), _p(ids), _p(wts)
+    r.expert_offsets, r.sorted_pair, r.pair_pos = _p(offsets), _p(sorted_pair), _p(pair_pos)
+    r.num_tokens, r.num_experts, r.top_k, r.hidden, r.act_dtype, r.scale, r.x_stride_t = T, E, top_k, H, _act(x), route_scale, x.stride(0)
+    _C.check(lib.hymeta_moe_route_sigmoid(C.byref(r), st), "hymeta_moe_route_sigmoid")
+
+    if (x.dtype == torch.bfloat16 and moe_mfma_shapes(H, inter) and E <= 64 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0):
+        h13 = torch.empty(P, two_i, dtype=torch.bfloat16, device=dev)
+        g = _C.MoeGemmArgs()
+        g.x, g.weights, g.out, g.expert_offsets = _p(x), _p(w13), _p(h13), _p(offsets)
+        g.a_rows, g.a_rows_div, g.max_rows, g.K, g.N = _p(sorted_pair), top_k, P, H, two_i
+        g.local_expert_begin, g.local_expert_end = 0, E
+        g.x_stride_m, g.out_stride_m, g.w_stride_e = x.stride(0), h13.stride(0), w13.stride(0)
+        _C.check(lib.hymeta_moe_gemm(C.byref(g), st), "hymeta_moe_gemm (w13)")
+        hact = clamped_glu(h13, limit, alpha)
+        y = torch.empty(P, H, dtype=torch.bfloat16, device=dev)
+        d = _C.MoeGemmArgs()
+        d.x, d.x_stride_m, d.weights, d.out, d.expert_offsets = _p(hact), hact.stride(0), _p(w2), _p(y), _p(offsets)
+        d.scale_rows, d.row_scale = _p(sorted_pair), _p(wts)
+        d.a_rows_div, d.max_rows, d.K, d.N = 1, P, inter, H
+        d.local_expert_begin, d.local_expert_end = 0, E
+        d.out_stride_m, d.w_stride_e = y.stride(0), w2.stride(0)
+        _C.check(lib.hymeta_moe_gemm(C.byref(d), st), "hymeta_moe_gemm (w2)")
+        c = _C.MoeCombineArgs()
+        c.y, c.out, c.pair_pos, c.topk_weights = _p(y), _p(out), _p(pair_pos), _p(wts)
+        c.num_tokens, c.hidden, c.top_k = T, H, top_k
+        c.y_stride_m, c.out_stride_m = y.stride(0), out.stride(0)
+        _C.check(lib.hymeta_moe_combine(C.byref(c), st), "hymeta_moe_combine")
+        return out
+
+    act = _DT[x.dtype]
+    hact = torch.empty(P, inter, dtype=x.dtype, device=dev)
+    g = _C.MoeGemmAnyArgs()
+    g.x, g.weights, g.out, g.expert_offsets = _p(x), _p(w13), _p(hact), _p(offsets)
+    g.a_rows, g.a_rows_div, g.max_rows, g.K, g.N, g.num_experts, g.gated, g.act_dtype = _p(sorted_pair), top_k, P, H, inter, E, _C.GLU_CLAMPED, act
+    g.act_limit, g.act_alpha = limit, alpha
+    g.x_stride_m, g.out_stride_m, g.w_stride_e = x.stride(0), hact.stride(0), w13.stride(0)
+    _C.check(lib.hymeta_moe_gemm_any(C.byref(g), st), "hymeta_moe_gemm_any (w13)")
+    y = torch.empty(P, H, dtype=x.dtype, device=dev)
+    d = _C.MoeGemmAnyArgs()
+    d.x, d.weights, d.out, d.expert_offsets = _p(hact), _p(w2), _p(y), _p(offsets)
+    d.scale_rows, d.row_scale = _p(sorted_pair), _p(wts)
+    d.a_rows_div, d.max_rows, d.K, d.N, d.num_experts, d.gated, d.act_dtype = 1, P, inter, H, E, _C.GLU_NONE, act
+    d.x_stride_m, d.out_stride_m, d.w_stride_e = hact.stride(0), y.stride(0), w2.stride(0)
+    _C.check(lib.hymeta_moe_gemm_any(C.byref(d), st), "hymeta_moe_gemm_any (w2)")
+    c = _C.MoeCombineAnyArgs()
+    c.y, c.out, c.pair_pos = _p(y), _p(out), _p(pair_pos)
+    c.num_tokens, c.width, c.top_k, c.act_dtype = T, H, top_k, act
     c.y_stride_m, c.out_stride_m = y.stride(0), out.stride(0)
     _C.check(lib.hymeta_moe_combine_any(C.byref(c), st), "hymeta_moe_combine_any")
     return out

@@ -1,0 +1,62 @@
+"""Feed-forward sublayers of the post-norm designs:
+
+``XieluMLP``        ``W_down xielu(W_up h + b_up) + b_down`` with ``xielu(z) = a_pos z^2 + z / 2`` for ``z > 0`` and
+                    ``a_neg (exp(z) - 1 - z) + z / 2`` otherwise, ``a_pos = softplus(p)``, ``a_neg = 1/2 + softplus(q)``
+``ClampedGluMLP``   ``W_down (g sigmoid(alpha g) (u + 1))`` with ``g = min(W_gate h, limit)``, ``u = clamp(W_up h, +-limit)``
+``SigmoidRoutedMoE``  experts of the second form chosen by the largest ``sigmoid`` router scores, weighing their scores
+                    over the chosen's sum times a constant, beside an optional shared expert that every token runs
+
+Beside ``HymetaMoE`` (``moe.py``: softmax router, silu experts) and ``TableMoE`` (``table_moe.py``: no router network);
+the expert stacks ``w13 [E, 2I, H]`` / ``w2 [E, H, I]`` are theirs.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from .. import hip_ops
+from ..linear import HymetaLinear
+
+GLU_ALPHA = 1.702       # the sigmoid's slope in the clamped gated unit
+
+
+def _softplus(v: float) -> float:
+    return max(v, 0.0) + math.log1p(math.exp(-abs(v)))
+
+
+class XieluMLP(torch.nn.Module):
+    def __init__(self, up_proj: HymetaLinear, down_proj: HymetaLinear, p: float, q: float):
+        super().__init__()
+        self.up_proj, self.down_proj = up_proj, down_proj
+        self.a_pos, self.a_neg = _softplus(float(p)), 0.5 + _softplus(float(q))
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return self.down_proj(hip_ops.xielu(self.up_proj(h), self.a_pos, self.a_neg))
+
+
+class ClampedGluMLP(torch.nn.Module):
+    def __init__(self, gate_up_proj: HymetaLinear, down_proj: HymetaLinear, limit: float, alpha: float = GLU_ALPHA):
+        """``gate_up_proj``: rows = gate, then up."""
+        super().__init__()
+        self.gate_up_proj, self.down_proj, self.limit, self.alpha = gate_up_proj, down_proj, float(limit), float(alpha)
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        return self.down_proj(hip_ops.clamped_glu(self.gate_up_proj(h), self.limit, self.alpha))
+
+
+class SigmoidRoutedMoE(torch.nn.Module):
+    def __init__(self, router_weight: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, top_k: int, route_scale: float, limit: float,
+                 shared: Optional[ClampedGluMLP] = None, alpha: float = GLU_ALPHA):
+        super().__init__()
+        self.register_buffer("router_weight", router_weight.float().contiguous())     # the router runs in fp32
+        self.register_buffer("w13", w13.contiguous())
+        self.register_buffer("w2", w2.contiguous())
+        self.top_k, self.route_scale, self.limit, self.alpha, self.shared = int(top_k), float(route_scale), float(limit), float(alpha), shared
+
+    def forward(self, h: torch.Tensor) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        """``(routed experts' weighted sum, shared expert's output or None)``: whoever adds them to the stream adds both."""
+        y = hip_ops.moe_sigmoid_forward(h, self.router_weight, self.w13, self.w2, self.top_k, self.route_scale, self.limit, self.alpha)
+        return y, (None if self.shared is None else self.shared(h))

@@ -21,6 +21,11 @@ def _sonuzen_config(model_dir: str):
     return SonuzenConfig.from_pretrained(model_dir)
 
 
+def _geponex_config(model_dir: str):
+    from .models.configuration_geponex import GeponexConfig
+    return GeponexConfig.from_pretrained(model_dir)
+
+
 def _gla_swa_config(model_dir: str):
     from .model_for_7B.configuration_gla_swa import GLAswaConfig
     with open(os.path.join(model_dir, "config.json")) as f:
@@ -31,6 +36,8 @@ def _gla_swa_config(model_dir: str):
 
 register("Sonuzen", "vllm_hymeta.models.modeling_sonuzen:SonuzenForCausalLM", _sonuzen_config)
 register("SonuzenForCausalLM", "vllm_hymeta.models.modeling_sonuzen:SonuzenForCausalLM", _sonuzen_config)
+register("Geponex", "vllm_hymeta.models.modeling_geponex:GeponexForCausalLM", _geponex_config)
+register("GeponexForCausalLM", "vllm_hymeta.models.modeling_geponex:GeponexForCausalLM", _geponex_config)
 register("GLAswaForCausalLM", "vllm_hymeta.model_for_7B.modeling_gla_swa:GLAswaForCausalLM", _gla_swa_config)
 
 
@@ -60,6 +67,8 @@ def kernel_sources(model_dir: str):
 _KERNEL_SOURCES = {
     "SonuzenForCausalLM": ("api_misc", "norm_conv", "mingru", "sink_attn", "moe_table", "moe", "glue", "dense_gemm", "stream_gemm",
                            "tall_gemm"),
+    "GeponexForCausalLM": ("api_misc", "norm_conv", "post_norm", "latent_attn", "sink_attn", "lightning", "gated_ops", "moe_sigmoid",
+                           "moe_table", "moe", "glue", "dense_gemm", "stream_gemm", "tall_gemm"),
 }
 
 
