@@ -265,3 +265,18 @@ def geponex_random_weights(cfg: dict, seed: int = 0, std: float = 1.0) -> Dict[s
                 Fs = mlp["shared"]["ff"]
                 w[p + "mlp.shared.gate"], w[p + "mlp.shared.up"], w[p + "mlp.shared.down"] = lin(Fs, W), lin(Fs, W), lin(W, Fs)
     return w
+
+
+def shared_row_attention_ref(q: torch.Tensor, rows: torch.Tensor, v_dim: int, scale: float, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal attention of ``q [T, H, Dk]`` over ``rows [T, Dk]`` that all heads share as keys, the first ``v_dim`` elements
+    of a row being its value; ``sink [H]``: a logit per head in the denominator.  -> ``[T, H, v_dim]``."""
+    T, H, _ = q.shape
+    out = torch.zeros(T, H, v_dim, dtype=q.dtype)
+    for h in range(H):
+        for i in range(T):
+            s = (rows[:i + 1] @ q[i, h]) * scale
+            mx = s.max() if sink is None else torch.maximum(s.max(), sink[h])
+            e = torch.exp(s - mx)
+            den = e.sum() + (0 if sink is None else torch.exp(sink[h] - mx))
+            out[i, h] = (e / den) @ rows[:i + 1, :v_dim]
+    return out
