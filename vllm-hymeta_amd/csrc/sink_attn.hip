@@ -176,12 +176,15 @@ struct MfmaSmem {
 // the same 8 channels of 4 consecutive keys (4 chunks), which are 8 runs of 4 keys in the transposed image, one 8-byte
 // store each.  The 4-key groups of a channel are permuted by the channel's chunk number (XOR), which spreads the stores
 // of threads that hold the same keys over the banks; the reader applies the same permutation.
-template <int D, int DV, int Threads>
+// VinK: a head's part of a cache row is its key alone (D elements), whose first DV elements are also its value.
+template <int D, int DV, int Threads, bool VinK>
 struct TileStage {
   static constexpr int kKeyChunksPerRow = D / 8, kValChunksPerRow = DV / 8;
-  static constexpr int kKeyPerThread = kTileKeys * kKeyChunksPerRow / Threads;
+  static constexpr int kKeyChunks = kTileKeys * kKeyChunksPerRow;
+  static constexpr int kKeyPerThread = (kKeyChunks + Threads - 1) / Threads;
   static constexpr int kValBlocks = (kTileKeys / 4) * kValChunksPerRow;       // (4 keys) x (8 channels) each
-  static_assert(kTileKeys * kKeyChunksPerRow % Threads == 0 && kValBlocks <= Threads, "the staging roles fit the workgroup");
+  static constexpr int kHeadElems = VinK ? D : D + DV, kValueAt = VinK ? 0 : D;
+  static_assert(D % 32 == 0 && DV % 16 == 0 && kValBlocks <= Threads && (!VinK || DV <= D), "the staging roles fit the workgroup");
   u32x4 rk[kKeyPerThread];
   u32x4 rv[4];
 
@@ -201,8 +204,8 @@ struct TileStage {
     Pages p;
     p.cache = static_cast<const uint16_t*>(a.kv_cache);
     p.bt = bt;
-    p.row_elems = static_cast<int64_t>(a.num_kv_heads) * (D + DV);
-    p.head_off = static_cast<int64_t>(g) * (D + DV);
+    p.row_elems = static_cast<int64_t>(a.num_kv_heads) * kHeadElems;
+    p.head_off = static_cast<int64_t>(g) * kHeadElems;
     p.shift = __builtin_ctz(a.block_size);
     p.mask = a.block_size - 1;
     p.whole = a.block_size >= kTileKeys;
@@ -223,7 +226,7 @@ struct TileStage {
       const int idx = i * Threads + threadIdx.x;
       const int j = j0 + idx / kKeyChunksPerRow;
       rk[i] = u32x4{0u, 0u, 0u, 0u};
-      if (j <= last) rk[i] = ld16g(row_ptr(p, j0, j) + (idx % kKeyChunksPerRow) * 8);
+      if (j <= last && (kKeyChunks % Threads == 0 || idx < kKeyChunks)) rk[i] = ld16g(row_ptr(p, j0, j) + (idx % kKeyChunksPerRow) * 8);
     }
     if (static_cast<int>(threadIdx.x) < kValBlocks) {
       const int ch = threadIdx.x % kValChunksPerRow, grp = threadIdx.x / kValChunksPerRow;
@@ -231,7 +234,7 @@ struct TileStage {
       for (int i = 0; i < 4; ++i) {
         const int j = j0 + 4 * grp + i;
         rv[i] = u32x4{0u, 0u, 0u, 0u};
-        if (j <= last) rv[i] = ld16g(row_ptr(p, j0, j) + D + ch * 8);
+        if (j <= last) rv[i] = ld16g(row_ptr(p, j0, j) + kValueAt + ch * 8);
       }
     }
   }
@@ -240,7 +243,8 @@ struct TileStage {
 #pragma unroll
     for (int i = 0; i < kKeyPerThread; ++i) {
       const int idx = i * Threads + threadIdx.x;
-      st16(&sm.k[(idx / kKeyChunksPerRow) * MfmaSmem<D, DV>::kPitchK + (idx % kKeyChunksPerRow) * 8], rk[i]);
+      if (kKeyChunks % Threads == 0 || idx < kKeyChunks)
+        st16(&sm.k[(idx / kKeyChunksPerRow) * MfmaSmem<D, DV>::kPitchK + (idx % kKeyChunksPerRow) * 8], rk[i]);
     }
     if (static_cast<int>(threadIdx.x) < kValBlocks) {
       const int ch = threadIdx.x % kValChunksPerRow, grp = threadIdx.x / kValChunksPerRow;
@@ -399,7 +403,7 @@ template <int RB> struct PrefillShape { static constexpr int kRows = 16 * RB * k
 
 // Portions of prompts: grid = (tiles of 128 RB rows, heads, sequences); a wave holds RB blocks of 16 rows; sequences with
 // one row are left to the decode form.
-template <int D, int DV, int RB>
+template <int D, int DV, int RB, bool VinK>
 __global__ __launch_bounds__(64 * kPrefillWaves) void sink_attention_prefill_mfma_kernel(hymeta_sink_attention_args a) {
   constexpr int kRows = PrefillShape<RB>::kRows;
   __shared__ MfmaSmem<D, DV> sm[2];
@@ -432,7 +436,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void sink_attention_prefill_mfm
   if (a.window_left >= 0) j_first = max(0, ctx + static_cast<int>(blockIdx.x) * kRows - a.window_left) / kTileKeys * kTileKeys;
   // two LDS images: while the waves multiply tile t out of one, tile t + 1 goes into the other and the loads of tile
   // t + 2 are in flight; one barrier per tile
-  TileStage<D, DV, 64 * kPrefillWaves> stage;
+  TileStage<D, DV, 64 * kPrefillWaves, VinK> stage;
   stage.issue(a, bt, g, j_first, block_last);
   stage.commit(sm[0]);
   if (j_first + kTileKeys <= block_last) stage.issue(a, bt, g, j_first + kTileKeys, block_last);
@@ -473,7 +477,7 @@ constexpr int kDecodeWaves = 4;
 // Decode: a workgroup per (sequence with one row, key/value head, slice of the keys); rows = the group's query heads; the
 // four waves share the staged tiles and take a 16-key subtile each.  Every wave writes its (maximum, denominator,
 // weighted values) per head; the combine kernel merges them and the sink.
-template <int D, int DV, int RB>
+template <int D, int DV, int RB, bool VinK>
 __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_kernel(hymeta_sink_attention_args a, int splits, int tiles_per_split) {
   __shared__ MfmaSmem<D, DV> sm[2];
   const int s = blockIdx.z, g = blockIdx.y, split = blockIdx.x;
@@ -505,7 +509,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
     for (int cb = 0; cb < DV / 16; ++cb) w.o[rb][cb] = f32x4v{0.f, 0.f, 0.f, 0.f};
   }
   if (j_lo < first) j_lo = first / kTileKeys * kTileKeys;      // tiles wholly before the window are not read
-  TileStage<D, DV, 64 * kDecodeWaves> stage;
+  TileStage<D, DV, 64 * kDecodeWaves, VinK> stage;
   if (j_lo <= j_hi) {
     stage.issue(a, bt, g, j_lo, j_hi);
     stage.commit(sm[0]);
@@ -568,10 +572,13 @@ __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymet
   }
 }
 
+// Head sizes the matrix-core kernels are built for.  A value inside its key: a latent of 64 or 128 followed by a rotated
+// part of 32 or 64.
 inline bool mfma_shape(const hymeta_sink_attention_args& a) {
-  const bool dims = (a.head_dim == 64 || a.head_dim == 128) && (a.v_dim == 64 || a.v_dim == 128);
-  return a.act_dtype == HYMETA_BF16 && dims && a.kv_layout == HYMETA_KV_KEY_THEN_VALUE && a.num_heads / a.num_kv_heads <= kRowsPerWave &&
-         a.q_stride_t % 8 == 0 &&
+  bool dims = (a.head_dim == 64 || a.head_dim == 128) && (a.v_dim == 64 || a.v_dim == 128);
+  if (a.kv_layout == HYMETA_KV_VALUE_IN_KEY)
+    dims = (a.v_dim == 64 || a.v_dim == 128) && (a.head_dim == a.v_dim + 32 || a.head_dim == a.v_dim + 64);
+  return a.act_dtype == HYMETA_BF16 && dims && a.num_heads / a.num_kv_heads <= kRowsPerWave && a.q_stride_t % 8 == 0 &&
          (a.block_size & (a.block_size - 1)) == 0 &&
          (reinterpret_cast<uintptr_t>(a.q) | reinterpret_cast<uintptr_t>(a.kv_cache) | reinterpret_cast<uintptr_t>(a.out)) % 16 == 0;
 }
@@ -583,12 +590,12 @@ inline int decode_splits(int num_seqs, int num_kv_heads, int max_seq_len) {
   return splits > tiles ? (tiles < 1 ? 1 : tiles) : splits;
 }
 
-template <int D, int DV>
+template <int D, int DV, bool VinK = false>
 int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st) {
   if (a.max_query_len > 1) {
     constexpr int kRB = PREFILL_RB;
     const dim3 grid((a.max_query_len + PrefillShape<kRB>::kRows - 1) / PrefillShape<kRB>::kRows, a.num_heads, a.num_seqs);
-    hipLaunchKernelGGL((sink_attention_prefill_mfma_kernel<D, DV, kRB>), grid, dim3(64 * kPrefillWaves), 0, st, a);
+    hipLaunchKernelGGL((sink_attention_prefill_mfma_kernel<D, DV, kRB, VinK>), grid, dim3(64 * kPrefillWaves), 0, st, a);
   }
   // sequences with a single row: every step but a pure prompt step has some; a prompt of one token is one too
   const int splits = decode_splits(a.num_seqs, a.num_kv_heads, a.max_seq_len);
@@ -596,9 +603,9 @@ int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st) {
   const int tiles_per_split = (tiles + splits - 1) / splits;
   const dim3 grid(splits, a.num_kv_heads, a.num_seqs);
   if (a.num_heads / a.num_kv_heads <= 16)
-    hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 1>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split);
+    hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 1, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split);
   else
-    hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 2>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split);
+    hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 2, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split);
   hipLaunchKernelGGL(sink_attention_decode_combine_kernel, dim3(a.num_seqs, a.num_heads), dim3(64), 0, st, a, splits);
   return launch_status();
 }
@@ -654,6 +661,10 @@ extern "C" int hymeta_sink_attention(const hymeta_sink_attention_args* args, hym
     const size_t need = hymeta_sink_attention_workspace_bytes(a.num_seqs, a.num_heads, a.num_kv_heads, a.v_dim, a.max_seq_len);
     if (!a.workspace || a.workspace_bytes < need) return HYMETA_ERR_WORKSPACE;
     if (a.num_seqs > 65535 || a.num_heads > 65535) return HYMETA_ERR_UNSUPPORTED;
+    if (a.kv_layout == HYMETA_KV_VALUE_IN_KEY) {
+      if (a.v_dim == 64) return a.head_dim == 96 ? launch_mfma<96, 64, true>(a, st) : launch_mfma<128, 64, true>(a, st);
+      return a.head_dim == 160 ? launch_mfma<160, 128, true>(a, st) : launch_mfma<192, 128, true>(a, st);
+    }
     if (a.head_dim == 64 && a.v_dim == 64) return launch_mfma<64, 64>(a, st);
     if (a.head_dim == 64 && a.v_dim == 128) return launch_mfma<64, 128>(a, st);
     if (a.head_dim == 128 && a.v_dim == 64) return launch_mfma<128, 64>(a, st);
