@@ -1336,8 +1336,9 @@ int hymeta_latent_q_assemble(const hymeta_latent_q_assemble_args* args, hymeta_s
  *   q, k, v = silu of the columns [0, H D), [H D, 2 H D), [2 H D, 2 H D + H Dv) of qkv
  *   S <- decay[h] S + k v^T,   out = S^T q        (S fp32 [head_dim, v_dim] per sequence and head)
  * state fp32 [slots, H, head_dim, v_dim] is read where context_lens > 0 (else the state starts at zero) and written.
- * Portions of at least HYMETA_LIGHTNING_CHUNK rows of bf16 activations with head_dim and v_dim multiples of 32 up to 128
- * run in chunks on the matrix cores; everything else token by token. */
+ * Portions of 8 rows or more of bf16 activations with head_dim 32, 64 or 128 and v_dim a multiple of 32 run in chunks of
+ * HYMETA_LIGHTNING_CHUNK rows on the matrix cores (the state stays fp32; what enters a product from fp32 goes in as two
+ * bf16 parts); everything else token by token. */
 #define HYMETA_LIGHTNING_CHUNK 64
 typedef struct hymeta_lightning_attention_args {
   uint32_t struct_size;

@@ -11,14 +11,14 @@ __device__ __forceinline__ float silu_f(float x) { return x / (1.f + expf(-x)); 
 // Token by token.  grid = (heads, sequences, value columns in runs of 256); a thread owns one value column c and keeps
 // that column of the state, S[:, c], in registers; q_t and k_t go through LDS.
 template <typename A, int DMAX>
-__global__ __launch_bounds__(256) void lightning_rows_kernel(hymeta_lightning_attention_args a) {
+__global__ __launch_bounds__(256) void lightning_rows_kernel(hymeta_lightning_attention_args a, int max_rows) {
   typedef typename A::elem elem;
   __shared__ float s_q[2][DMAX], s_k[2][DMAX];
   const int h = blockIdx.x, s = blockIdx.y;
   const int c = blockIdx.z * 256 + threadIdx.x;
   const int H = a.num_heads, D = a.head_dim, Dv = a.v_dim;
   const int r0 = a.query_start_loc[s], r1 = a.query_start_loc[s + 1];
-  if (r1 <= r0) return;
+  if (r1 <= r0 || r1 - r0 > max_rows) return;          // longer portions: the chunked kernel's
   const int slot = a.slot_idx[s];
   const bool live = c < Dv;
   float* st = (slot >= 0) ? a.state + ((static_cast<int64_t>(slot) * H + h) * D) * Dv : nullptr;
@@ -70,14 +70,204 @@ __global__ __launch_bounds__(256) void gated_rms_norm_kernel(hymeta_gated_rms_no
   for (int c = threadIdx.x; c < a.width; c += 256) A::st(out + c, x[c] * inv * a.weight[c] * sigmoid_exact(A::ld(g + c)));
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// bf16 portions in chunks of 64 rows on the matrix cores.  With S the state before the chunk, i and j rows of the
+// chunk, n its number of rows and L = decay:
+//   o_i   = L^(i+1) S^T q_i + sum_{j <= i} L^(i-j) (q_i . k_j) v_j
+//   S_new = L^n S + sum_j L^(n-1-j) k_j v_j^T
+// grid = (heads, sequences, value columns in slices of 32); 4 waves, each with 16 rows of the chunk.  The state
+// slice stays fp32 in registers, transposed (S^T [c][d]: a lane holds 4 value columns of one d), 16 x 16 blocks dealt
+// over the waves; what enters a matrix product from fp32 (the decayed weights, the decayed keys, the state) goes in as
+// hi + lo bf16 parts, two products, so that it keeps 16 bits of mantissa.
+// ------------------------------------------------------------------------------------------------
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+constexpr int kChunk = HYMETA_LIGHTNING_CHUNK, kSliceV = 32;
+constexpr int kChunkMinRows = 8;            // shorter portions go token by token
+
+__device__ __forceinline__ f32x4v mfma16(bf16x8 a, bf16x8 b, f32x4v c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+
+__device__ __forceinline__ float decay_pow(float log2_decay, int x) { return x == 0 ? 1.f : exp2f(static_cast<float>(x) * log2_decay); }
+
+// 8 bf16 of a row through silu, back to bf16 (and, optionally, the fp32 values)
+__device__ __forceinline__ u32x4 silu8(u32x4 raw, float* vals) {
+  u32x4 out;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float lo = silu_f(bf2f(static_cast<uint16_t>(raw[e] & 0xffffu))), hi = silu_f(bf2f(static_cast<uint16_t>(raw[e] >> 16)));
+    if (vals) vals[2 * e] = lo, vals[2 * e + 1] = hi;
+    out[e] = pack_bf16x2(lo, hi);
+  }
+  return out;
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void lightning_chunk_kernel(hymeta_lightning_attention_args a, int min_rows) {
+  constexpr int PK = D + 8, PT = kChunk + 8, NBW = (2 * D / 16) / 4;
+  __shared__ __attribute__((aligned(16))) uint16_t sk[kChunk * PK];          // silu(k), a row per key
+  __shared__ __attribute__((aligned(16))) uint16_t skt[2][D * PT];           // decayed keys, transposed [d][key], hi / lo
+  __shared__ __attribute__((aligned(16))) uint16_t svt[kSliceV * PT];        // silu(v) of the slice, transposed [c][key]
+  __shared__ __attribute__((aligned(16))) uint16_t sst[2][kSliceV * PK];     // state^T [c][d], hi / lo
+  const int h = blockIdx.x, s = blockIdx.y, vs = blockIdx.z;
+  const int r0 = a.query_start_loc[s], rows = a.query_start_loc[s + 1] - r0;
+  if (rows < min_rows) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, g4 = lane >> 4;
+  const int H = a.num_heads, Dv = a.v_dim;
+  const int slot = a.slot_idx[s];
+  float* st = slot >= 0 ? a.state + ((static_cast<int64_t>(slot) * H + h) * D) * Dv + vs * kSliceV : nullptr;
+  const float decay = a.decay[h];
+  const float l2 = decay > 0.f ? log2f(decay) : -INFINITY;
+  const bool carry = st != nullptr && a.context_lens[s] > 0;
+  f32x4v S[NBW];
+#pragma unroll
+  for (int ib = 0; ib < NBW; ++ib) {
+    const int b = wave + 4 * ib, cb = b & 1, db = b >> 1;
+    S[ib] = carry ? *reinterpret_cast<const f32x4v*>(st + static_cast<int64_t>(16 * db + n) * Dv + 16 * cb + 4 * g4) : f32x4v{0.f, 0.f, 0.f, 0.f};
+  }
+  auto state_to_lds = [&]() {
+#pragma unroll
+    for (int ib = 0; ib < NBW; ++ib) {
+      const int b = wave + 4 * ib, cb = b & 1, db = b >> 1;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float v = S[ib][r];
+        const uint16_t hi = f2bf(v);
+        const int at = (16 * cb + 4 * g4 + r) * PK + 16 * db + n;
+        sst[0][at] = hi;
+        sst[1][at] = f2bf(v - bf2f(hi));
+      }
+    }
+  };
+  state_to_lds();
+  const uint16_t* qkv = static_cast<const uint16_t*>(a.qkv);
+  const int64_t q_off = static_cast<int64_t>(h) * D, k_off = static_cast<int64_t>(H) * D + q_off;
+  const int64_t v_off = 2 * static_cast<int64_t>(H) * D + static_cast<int64_t>(h) * Dv + vs * kSliceV;
+  for (int c0 = 0; c0 < rows; c0 += kChunk) {
+    const int nrow = min(kChunk, rows - c0);
+    const uint16_t* base = qkv + static_cast<int64_t>(r0 + c0) * a.qkv_stride_t;
+    for (int idx = tid; idx < kChunk * (D / 8); idx += 256) {
+      const int j = idx / (D / 8), ch = idx % (D / 8);
+      float vals[8];
+      u32x4 packed = u32x4{0u, 0u, 0u, 0u};
+      if (j < nrow) packed = silu8(ld16g(base + j * a.qkv_stride_t + k_off + 8 * ch), vals);
+      st16(&sk[j * PK + 8 * ch], packed);
+      const float kd = j < nrow ? decay_pow(l2, nrow - 1 - j) : 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float x = j < nrow ? vals[e] * kd : 0.f;
+        const uint16_t hi = f2bf(x);
+        skt[0][(8 * ch + e) * PT + j] = hi;
+        skt[1][(8 * ch + e) * PT + j] = f2bf(x - bf2f(hi));
+      }
+    }
+    for (int idx = tid; idx < kChunk * (kSliceV / 8); idx += 256) {
+      const int j = idx / (kSliceV / 8), ch = idx % (kSliceV / 8);
+      u32x4 packed = u32x4{0u, 0u, 0u, 0u};
+      if (j < nrow) packed = silu8(ld16g(base + j * a.qkv_stride_t + v_off + 8 * ch), nullptr);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) svt[(8 * ch + e) * PT + j] = static_cast<uint16_t>(e & 1 ? packed[e >> 1] >> 16 : packed[e >> 1] & 0xffffu);
+    }
+    __syncthreads();
+    const int i = 16 * wave + n;                       // this lane's row of the chunk (as a column of the products)
+    bf16x8 q[D / 32];
+#pragma unroll
+    for (int sd = 0; sd < D / 32; ++sd) {
+      u32x4 packed = u32x4{0u, 0u, 0u, 0u};
+      if (i < nrow) packed = silu8(ld16g(base + i * a.qkv_stride_t + q_off + 32 * sd + 8 * g4), nullptr);
+      q[sd] = __builtin_bit_cast(bf16x8, packed);
+    }
+    // weights of the chunk's own rows: (q_i . k_j) L^(i-j) for j <= i, as hi + lo parts
+    uint32_t phi[4][2], plo[4][2];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      f32x4v sc = f32x4v{0.f, 0.f, 0.f, 0.f};
+      if (ks <= wave) {
+#pragma unroll
+        for (int sd = 0; sd < D / 32; ++sd)
+          sc = mfma16(__builtin_bit_cast(bf16x8, ld16(&sk[(16 * ks + n) * PK + 32 * sd + 8 * g4])), q[sd], sc);
+      }
+      float p[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int j = 16 * ks + 4 * g4 + r;
+        p[r] = (ks <= wave && j <= i) ? sc[r] * decay_pow(l2, i - j) : 0.f;
+      }
+#pragma unroll
+      for (int r2 = 0; r2 < 2; ++r2) {
+        const uint32_t hi = pack_bf16x2(p[2 * r2], p[2 * r2 + 1]);
+        phi[ks][r2] = hi;
+        plo[ks][r2] = pack_bf16x2(p[2 * r2] - lo_bf(hi), p[2 * r2 + 1] - hi_bf(hi));
+      }
+    }
+    f32x4v o[2];
+    const float row_decay = decay_pow(l2, i + 1);
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+      // the state before the chunk
+      f32x4v x = f32x4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int sd = 0; sd < D / 32; ++sd) {
+        x = mfma16(__builtin_bit_cast(bf16x8, ld16(&sst[0][(16 * cb + n) * PK + 32 * sd + 8 * g4])), q[sd], x);
+        x = mfma16(__builtin_bit_cast(bf16x8, ld16(&sst[1][(16 * cb + n) * PK + 32 * sd + 8 * g4])), q[sd], x);
+      }
+      f32x4v acc = x * row_decay;
+#pragma unroll
+      for (int kp = 0; kp < 2; ++kp) {
+        if (2 * kp > wave) continue;
+        // k index 8 g4 + e of the product: keys 32 kp + 4 g4 + e for e < 4, 32 kp + 16 + 4 g4 + e - 4 after
+        const u32x2 v0 = *reinterpret_cast<const u32x2*>(&svt[(16 * cb + n) * PT + 32 * kp + 4 * g4]);
+        const u32x2 v1 = *reinterpret_cast<const u32x2*>(&svt[(16 * cb + n) * PT + 32 * kp + 16 + 4 * g4]);
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, (u32x4{v0[0], v0[1], v1[0], v1[1]}));
+        acc = mfma16(vf, __builtin_bit_cast(bf16x8, (u32x4{phi[2 * kp][0], phi[2 * kp][1], phi[2 * kp + 1][0], phi[2 * kp + 1][1]})), acc);
+        acc = mfma16(vf, __builtin_bit_cast(bf16x8, (u32x4{plo[2 * kp][0], plo[2 * kp][1], plo[2 * kp + 1][0], plo[2 * kp + 1][1]})), acc);
+      }
+      o[cb] = acc;
+    }
+    if (i < nrow) {
+      float* orow = a.out + static_cast<int64_t>(r0 + c0 + i) * H * Dv + static_cast<int64_t>(h) * Dv + vs * kSliceV;
+#pragma unroll
+      for (int cb = 0; cb < 2; ++cb) *reinterpret_cast<f32x4v*>(orow + 16 * cb + 4 * g4) = o[cb];
+    }
+    // the state after the chunk
+    const float chunk_decay = decay_pow(l2, nrow);
+#pragma unroll
+    for (int ib = 0; ib < NBW; ++ib) {
+      const int b = wave + 4 * ib, cb = b & 1, db = b >> 1;
+      f32x4v acc = S[ib] * chunk_decay;
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        const bf16x8 vf = __builtin_bit_cast(bf16x8, ld16(&svt[(16 * cb + n) * PT + 32 * kk + 8 * g4]));
+        acc = mfma16(vf, __builtin_bit_cast(bf16x8, ld16(&skt[0][(16 * db + n) * PT + 32 * kk + 8 * g4])), acc);
+        acc = mfma16(vf, __builtin_bit_cast(bf16x8, ld16(&skt[1][(16 * db + n) * PT + 32 * kk + 8 * g4])), acc);
+      }
+      S[ib] = acc;
+    }
+    __syncthreads();            // every wave is done with this chunk's tiles and with the old state's image
+    state_to_lds();             // (made visible by the barrier after the next chunk's staging)
+  }
+  if (st != nullptr) {
+#pragma unroll
+    for (int ib = 0; ib < NBW; ++ib) {
+      const int b = wave + 4 * ib, cb = b & 1, db = b >> 1;
+      *reinterpret_cast<f32x4v*>(st + static_cast<int64_t>(16 * db + n) * Dv + 16 * cb + 4 * g4) = S[ib];
+    }
+  }
+}
+
+inline bool chunk_shape(const hymeta_lightning_attention_args& a) {
+  return a.act_dtype == HYMETA_BF16 && (a.head_dim == 32 || a.head_dim == 64 || a.head_dim == 128) && a.v_dim % kSliceV == 0 &&
+         a.qkv_stride_t % 8 == 0 && reinterpret_cast<uintptr_t>(a.qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(a.state) % 16 == 0 &&
+         reinterpret_cast<uintptr_t>(a.out) % 16 == 0 && a.v_dim / kSliceV <= 65535;
+}
+
 template <typename A>
-void launch_rows(const hymeta_lightning_attention_args& a, hipStream_t st) {
+void launch_rows(const hymeta_lightning_attention_args& a, hipStream_t st, int max_rows) {
   const dim3 grid(a.num_heads, a.num_seqs, (a.v_dim + 255) / 256);
   const dim3 block(a.v_dim >= 256 ? 256 : (a.v_dim + 63) / 64 * 64);
-  if (a.head_dim <= 32) hipLaunchKernelGGL((lightning_rows_kernel<A, 32>), grid, block, 0, st, a);
-  else if (a.head_dim <= 64) hipLaunchKernelGGL((lightning_rows_kernel<A, 64>), grid, block, 0, st, a);
-  else if (a.head_dim <= 128) hipLaunchKernelGGL((lightning_rows_kernel<A, 128>), grid, block, 0, st, a);
-  else hipLaunchKernelGGL((lightning_rows_kernel<A, 256>), grid, block, 0, st, a);
+  if (a.head_dim <= 32) hipLaunchKernelGGL((lightning_rows_kernel<A, 32>), grid, block, 0, st, a, max_rows);
+  else if (a.head_dim <= 64) hipLaunchKernelGGL((lightning_rows_kernel<A, 64>), grid, block, 0, st, a, max_rows);
+  else if (a.head_dim <= 128) hipLaunchKernelGGL((lightning_rows_kernel<A, 128>), grid, block, 0, st, a, max_rows);
+  else hipLaunchKernelGGL((lightning_rows_kernel<A, 256>), grid, block, 0, st, a, max_rows);
 }
 
 }  // namespace
@@ -96,8 +286,16 @@ extern "C" int hymeta_lightning_attention(const hymeta_lightning_attention_args*
   if (!a.qkv || !a.state || !a.decay || !a.out || !a.query_start_loc || !a.context_lens || !a.slot_idx) return HYMETA_ERR_INVALID_ARG;
   if (a.qkv_stride_t < static_cast<int64_t>(a.num_heads) * (2 * a.head_dim + a.v_dim)) return HYMETA_ERR_INVALID_ARG;
   hipStream_t st = begin_launches(stream);
-  if (a.act_dtype == HYMETA_BF16) launch_rows<ActBf16>(a, st);
-  else launch_rows<ActF32>(a, st);
+  int max_rows = 0x7fffffff;
+  if (chunk_shape(a) && a.max_query_len >= kChunkMinRows) {
+    const dim3 grid(a.num_heads, a.num_seqs, a.v_dim / kSliceV);
+    if (a.head_dim == 32) hipLaunchKernelGGL(lightning_chunk_kernel<32>, grid, dim3(256), 0, st, a, kChunkMinRows);
+    else if (a.head_dim == 64) hipLaunchKernelGGL(lightning_chunk_kernel<64>, grid, dim3(256), 0, st, a, kChunkMinRows);
+    else hipLaunchKernelGGL(lightning_chunk_kernel<128>, grid, dim3(256), 0, st, a, kChunkMinRows);
+    max_rows = kChunkMinRows - 1;
+  }
+  if (a.act_dtype == HYMETA_BF16) launch_rows<ActBf16>(a, st, max_rows);
+  else launch_rows<ActF32>(a, st, max_rows);
   return launch_status();
 }
 
