@@ -23,13 +23,27 @@ __global__ __launch_bounds__(256) void activation_kernel(hymeta_activation_args 
   for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
     const elem* x = static_cast<const elem*>(a.x) + r * a.x_stride;
     elem* out = static_cast<elem*>(a.out) + r * a.out_stride;
-    if (a.kind == HYMETA_ACT_CLAMPED_GLU) {
-      for (int c = threadIdx.x; c < a.n; c += 256) A::st(out + c, clamped_glu(A::ld(x + c), A::ld(x + a.n + c), a.p0, a.p1));
-    } else if (a.kind == HYMETA_ACT_XIELU) {
-      for (int c = threadIdx.x; c < a.n; c += 256) A::st(out + c, xielu(A::ld(x + c), a.p0, a.p1));
-    } else {
-      const elem* g = static_cast<const elem*>(a.gate) + r * a.gate_stride;
-      for (int c = threadIdx.x; c < a.n; c += 256) A::st(out + c, A::ld(x + c) * sigmoid_exact(A::ld(g + c)));
+    // four columns a round, their loads in flight together
+    const elem* g = a.gate ? static_cast<const elem*>(a.gate) + r * a.gate_stride : nullptr;
+    for (int c0 = threadIdx.x; c0 < a.n; c0 += 4 * 256) {
+      float v0[4], v1[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = c0 + 256 * u;
+        const bool ok = c < a.n;
+        v0[u] = ok ? A::ld(x + c) : 0.f;
+        v1[u] = !ok ? 0.f : a.kind == HYMETA_ACT_CLAMPED_GLU ? A::ld(x + a.n + c) : a.kind == HYMETA_ACT_SIGMOID_MUL ? A::ld(g + c) : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = c0 + 256 * u;
+        if (c >= a.n) continue;
+        float v;
+        if (a.kind == HYMETA_ACT_CLAMPED_GLU) v = clamped_glu(v0[u], v1[u], a.p0, a.p1);
+        else if (a.kind == HYMETA_ACT_XIELU) v = xielu(v0[u], a.p0, a.p1);
+        else v = v0[u] * sigmoid_exact(v1[u]);
+        A::st(out + c, v);
+      }
     }
   }
 }

@@ -55,7 +55,10 @@ __global__ __launch_bounds__(256) void lightning_rows_kernel(hymeta_lightning_at
   }
 }
 
-template <typename A>
+// Rows of up to kGatedCached columns are read once (a thread keeps its columns in registers).
+constexpr int kGatedPerThread = 16, kGatedCached = 256 * kGatedPerThread;
+
+template <typename A, bool Cached>
 __global__ __launch_bounds__(256) void gated_rms_norm_kernel(hymeta_gated_rms_norm_args a) {
   typedef typename A::elem elem;
   __shared__ float red[4];
@@ -64,12 +67,29 @@ __global__ __launch_bounds__(256) void gated_rms_norm_kernel(hymeta_gated_rms_no
   const elem* g = static_cast<const elem*>(a.gate) + t * a.gate_stride_t;
   elem* out = static_cast<elem*>(a.out) + t * a.width;
   float ss = 0.f;
+  if (Cached) {
+    float xv[kGatedPerThread], gv[kGatedPerThread];
+#pragma unroll
+    for (int u = 0; u < kGatedPerThread; ++u) {
+      const int c = threadIdx.x + 256 * u;
+      xv[u] = c < a.width ? x[c] : 0.f;
+      gv[u] = c < a.width ? A::ld(g + c) : 0.f;
+      ss = fmaf(xv[u], xv[u], ss);
+    }
+    ss = block_sum<4>(ss, red);
+    const float inv = 1.f / sqrtf(ss / static_cast<float>(a.width) + a.eps);
+#pragma unroll
+    for (int u = 0; u < kGatedPerThread; ++u) {
+      const int c = threadIdx.x + 256 * u;
+      if (c < a.width) A::st(out + c, xv[u] * inv * a.weight[c] * sigmoid_exact(gv[u]));
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < a.width; c += 256) ss = fmaf(x[c], x[c], ss);
   ss = block_sum<4>(ss, red);
   const float inv = 1.f / sqrtf(ss / static_cast<float>(a.width) + a.eps);
   for (int c = threadIdx.x; c < a.width; c += 256) A::st(out + c, x[c] * inv * a.weight[c] * sigmoid_exact(A::ld(g + c)));
 }
-
 
 // ------------------------------------------------------------------------------------------------
 // bf16 portions in chunks of 64 rows on the matrix cores.  With S the state before the chunk, i and j rows of the
@@ -87,14 +107,19 @@ constexpr int kChunkMinRows = 8;            // shorter portions go token by toke
 
 __device__ __forceinline__ f32x4v mfma16(bf16x8 a, bf16x8 b, f32x4v c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
 
-__device__ __forceinline__ float decay_pow(float log2_decay, int x) { return x == 0 ? 1.f : exp2f(static_cast<float>(x) * log2_decay); }
+__device__ __forceinline__ float decay_pow(float log2_decay, int x) {
+  return x == 0 ? 1.f : __builtin_amdgcn_exp2f(static_cast<float>(x) * log2_decay);
+}
+
+// the hardware's exponential and reciprocal (about 1 ulp each): the inputs and the result are bf16
+__device__ __forceinline__ float silu_fast(float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
 
 // 8 bf16 of a row through silu, back to bf16 (and, optionally, the fp32 values)
 __device__ __forceinline__ u32x4 silu8(u32x4 raw, float* vals) {
   u32x4 out;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    const float lo = silu_f(bf2f(static_cast<uint16_t>(raw[e] & 0xffffu))), hi = silu_f(bf2f(static_cast<uint16_t>(raw[e] >> 16)));
+    const float lo = silu_fast(bf2f(static_cast<uint16_t>(raw[e] & 0xffffu))), hi = silu_fast(bf2f(static_cast<uint16_t>(raw[e] >> 16)));
     if (vals) vals[2 * e] = lo, vals[2 * e + 1] = hi;
     out[e] = pack_bf16x2(lo, hi);
   }
@@ -142,40 +167,66 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(hymeta_lightning_a
   const uint16_t* qkv = static_cast<const uint16_t*>(a.qkv);
   const int64_t q_off = static_cast<int64_t>(h) * D, k_off = static_cast<int64_t>(H) * D + q_off;
   const int64_t v_off = 2 * static_cast<int64_t>(H) * D + static_cast<int64_t>(h) * Dv + vs * kSliceV;
+  // the rows of a chunk as they come from memory: this thread's share of the keys (KPT groups of 8 columns of one row) and
+  // of the value slice, and this lane's query fragment; loaded a chunk ahead
+  constexpr int KPT = kChunk * (D / 8) / 256;
+  u32x4 rk[KPT], rv, rq[D / 32];
+  auto fetch = [&](int c0) {
+    const int nrow = min(kChunk, rows - c0);
+    const uint16_t* base = qkv + static_cast<int64_t>(r0 + c0) * a.qkv_stride_t;
+#pragma unroll
+    for (int u = 0; u < KPT; ++u) {
+      const int idx = tid + 256 * u, j = idx % kChunk, ch = idx / kChunk;
+      rk[u] = u32x4{0u, 0u, 0u, 0u};
+      if (j < nrow) rk[u] = ld16g(base + j * a.qkv_stride_t + k_off + 8 * ch);
+    }
+    {
+      const int j = tid % kChunk, ch = tid / kChunk;
+      rv = u32x4{0u, 0u, 0u, 0u};
+      if (j < nrow) rv = ld16g(base + j * a.qkv_stride_t + v_off + 8 * ch);
+    }
+    const int i = 16 * wave + n;
+#pragma unroll
+    for (int sd = 0; sd < D / 32; ++sd) {
+      rq[sd] = u32x4{0u, 0u, 0u, 0u};
+      if (i < nrow) rq[sd] = ld16g(base + i * a.qkv_stride_t + q_off + 32 * sd + 8 * g4);
+    }
+  };
+  static_assert(kChunk * (kSliceV / 8) == 256, "one group of the value slice per thread");
+  fetch(0);
   for (int c0 = 0; c0 < rows; c0 += kChunk) {
     const int nrow = min(kChunk, rows - c0);
     const uint16_t* base = qkv + static_cast<int64_t>(r0 + c0) * a.qkv_stride_t;
-    for (int idx = tid; idx < kChunk * (D / 8); idx += 256) {
-      const int j = idx / (D / 8), ch = idx % (D / 8);
+    (void)base;
+    // a wave's lanes hold 64 different rows of one 8-column group: the transposed 2-byte stores of a wave fall on
+    // consecutive addresses (a lane per key), the row-major 16-byte stores on different banks
+#pragma unroll
+    for (int u = 0; u < KPT; ++u) {
+      const int idx = tid + 256 * u, j = idx % kChunk, ch = idx / kChunk;
       float vals[8];
-      u32x4 packed = u32x4{0u, 0u, 0u, 0u};
-      if (j < nrow) packed = silu8(ld16g(base + j * a.qkv_stride_t + k_off + 8 * ch), vals);
+      u32x4 packed = silu8(rk[u], vals);            // rows past the portion were fetched as zeros: silu(0) = 0
       st16(&sk[j * PK + 8 * ch], packed);
       const float kd = j < nrow ? decay_pow(l2, nrow - 1 - j) : 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float x = j < nrow ? vals[e] * kd : 0.f;
+        const float x = vals[e] * kd;
         const uint16_t hi = f2bf(x);
         skt[0][(8 * ch + e) * PT + j] = hi;
         skt[1][(8 * ch + e) * PT + j] = f2bf(x - bf2f(hi));
       }
     }
-    for (int idx = tid; idx < kChunk * (kSliceV / 8); idx += 256) {
-      const int j = idx / (kSliceV / 8), ch = idx % (kSliceV / 8);
-      u32x4 packed = u32x4{0u, 0u, 0u, 0u};
-      if (j < nrow) packed = silu8(ld16g(base + j * a.qkv_stride_t + v_off + 8 * ch), nullptr);
+    {
+      const int j = tid % kChunk, ch = tid / kChunk;
+      const u32x4 packed = silu8(rv, nullptr);
 #pragma unroll
       for (int e = 0; e < 8; ++e) svt[(8 * ch + e) * PT + j] = static_cast<uint16_t>(e & 1 ? packed[e >> 1] >> 16 : packed[e >> 1] & 0xffffu);
     }
-    __syncthreads();
     const int i = 16 * wave + n;                       // this lane's row of the chunk (as a column of the products)
     bf16x8 q[D / 32];
 #pragma unroll
-    for (int sd = 0; sd < D / 32; ++sd) {
-      u32x4 packed = u32x4{0u, 0u, 0u, 0u};
-      if (i < nrow) packed = silu8(ld16g(base + i * a.qkv_stride_t + q_off + 32 * sd + 8 * g4), nullptr);
-      q[sd] = __builtin_bit_cast(bf16x8, packed);
-    }
+    for (int sd = 0; sd < D / 32; ++sd) q[sd] = __builtin_bit_cast(bf16x8, silu8(rq[sd], nullptr));
+    __syncthreads();
+    if (c0 + kChunk < rows) fetch(c0 + kChunk);        // in flight while this chunk is multiplied
     // weights of the chunk's own rows: (q_i . k_j) L^(i-j) for j <= i, as hi + lo parts
     uint32_t phi[4][2], plo[4][2];
 #pragma unroll
@@ -307,7 +358,13 @@ extern "C" int hymeta_gated_rms_norm(const hymeta_gated_rms_norm_args* args, hym
   if (a.num_tokens == 0) return HYMETA_OK;
   if (!a.x || !a.gate || !a.weight || !a.out || a.gate_stride_t < a.width) return HYMETA_ERR_INVALID_ARG;
   hipStream_t st = begin_launches(stream);
-  if (a.act_dtype == HYMETA_BF16) hipLaunchKernelGGL(gated_rms_norm_kernel<ActBf16>, dim3(a.num_tokens), dim3(256), 0, st, a);
-  else hipLaunchKernelGGL(gated_rms_norm_kernel<ActF32>, dim3(a.num_tokens), dim3(256), 0, st, a);
+  const bool cached = a.width <= kGatedCached;
+  if (a.act_dtype == HYMETA_BF16) {
+    if (cached) hipLaunchKernelGGL((gated_rms_norm_kernel<ActBf16, true>), dim3(a.num_tokens), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gated_rms_norm_kernel<ActBf16, false>), dim3(a.num_tokens), dim3(256), 0, st, a);
+  } else {
+    if (cached) hipLaunchKernelGGL((gated_rms_norm_kernel<ActF32, true>), dim3(a.num_tokens), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((gated_rms_norm_kernel<ActF32, false>), dim3(a.num_tokens), dim3(256), 0, st, a);
+  }
   return launch_status();
 }

@@ -9,32 +9,61 @@ namespace {
 
 constexpr int kSortThreads = 1024;
 
-// grid = tokens, 256 threads.  A wave per expert's dot product (lanes over the hidden size, a fixed order of
-// summation); then wave 0 picks the top_k: every lane scans the experts lane, lane + 64, ..., the wave reduces to the
-// largest score and, among equals, the lowest expert.
+// grid = tokens in fours, 256 threads.  The experts' dot products over the workgroup, eight experts and four tokens a
+// round (a weight is loaded once for the four tokens; the loads of a round are independent of each other; the partial
+// sums meet through the waves and LDS in a fixed order); then wave w picks the top_k of token w: every lane scans the
+// experts lane, lane + 64, ..., the wave reduces to the largest score and, among equals, the lowest expert.
+constexpr int kRouteTokens = 4;
+
 template <typename A>
 __global__ __launch_bounds__(256) void moe_scores_topk_kernel(hymeta_moe_route_sigmoid_args a) {
   typedef typename A::elem elem;
-  __shared__ float s_score[HYMETA_MOE_TABLE_MAX_EXPERTS];
-  __shared__ float s_top[HYMETA_MOE_TABLE_MAX_EXPERTS];
-  const int64_t t = blockIdx.x;
+  __shared__ float s_score[kRouteTokens][HYMETA_MOE_TABLE_MAX_EXPERTS];
+  __shared__ float s_top[kRouteTokens][HYMETA_MOE_TABLE_MAX_EXPERTS];
+  __shared__ float s_part[4][kRouteTokens][8];
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * kRouteTokens;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, E = a.num_experts;
-  const elem* x = static_cast<const elem*>(a.x) + t * a.x_stride_t;
-  for (int e = wave; e < E; e += 4) {
-    const float* w = a.router_weight + static_cast<int64_t>(e) * a.hidden;
-    float z = 0.f;
-    for (int k = lane; k < a.hidden; k += 64) z = fmaf(A::ld(x + k), w[k], z);
-    z = wave_sum(z);
-    if (lane == 0) s_score[e] = sigmoid_exact(z);
+  const int live = min(static_cast<int64_t>(kRouteTokens), a.num_tokens - t0);
+  const elem* x[kRouteTokens];
+#pragma unroll
+  for (int i = 0; i < kRouteTokens; ++i) x[i] = static_cast<const elem*>(a.x) + (t0 + min(i, live - 1)) * a.x_stride_t;
+  for (int e0 = 0; e0 < E; e0 += 8) {
+    float acc[kRouteTokens][8] = {};
+#pragma unroll 2
+    for (int k = threadIdx.x; k < a.hidden; k += 256) {
+      float xv[kRouteTokens], wv[8];
+#pragma unroll
+      for (int i = 0; i < kRouteTokens; ++i) xv[i] = A::ld(x[i] + k);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) wv[j] = a.router_weight[static_cast<int64_t>(min(e0 + j, E - 1)) * a.hidden + k];
+#pragma unroll
+      for (int i = 0; i < kRouteTokens; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = fmaf(xv[i], wv[j], acc[i][j]);
+    }
+#pragma unroll
+    for (int i = 0; i < kRouteTokens; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float v = wave_sum(acc[i][j]);
+        if (lane == 0) s_part[wave][i][j] = v;
+      }
+    __syncthreads();
+    if (threadIdx.x < kRouteTokens * 8) {
+      const int i = threadIdx.x >> 3, j = threadIdx.x & 7;
+      if (e0 + j < E) s_score[i][e0 + j] = sigmoid_exact((s_part[0][i][j] + s_part[1][i][j]) + (s_part[2][i][j] + s_part[3][i][j]));
+    }
+    __syncthreads();
   }
-  __syncthreads();
-  if (wave != 0) return;
+  if (wave >= live) return;
+  const int64_t t = t0 + wave;
+  float* score = s_score[wave];
   float total = 0.f;
   for (int k = 0; k < a.top_k; ++k) {
     float best = -2.f;
     int arg = 0x7fffffff;
     for (int e = lane; e < E; e += 64) {
-      const float v = s_score[e];
+      const float v = score[e];
       if (v > best) best = v, arg = e;            // ascending e: the first of equals stays
     }
     const float top = wave_max(best);
@@ -44,14 +73,14 @@ __global__ __launch_bounds__(256) void moe_scores_topk_kernel(hymeta_moe_route_s
     total += top;
     if (lane == 0) {
       a.topk_ids[t * a.top_k + k] = cand;
-      s_top[k] = top;
-      s_score[cand] = -1.f;                       // scores are >= 0: taken
+      s_top[wave][k] = top;
+      score[cand] = -1.f;                         // scores are >= 0: taken
     }
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
   }
   const float inv = a.scale / (total + 1e-20f);
-  for (int k = lane; k < a.top_k; k += 64) a.topk_weights[t * a.top_k + k] = s_top[k] * inv;
+  for (int k = lane; k < a.top_k; k += 64) a.topk_weights[t * a.top_k + k] = s_top[wave][k] * inv;
 }
 
 // One workgroup: count the pairs per expert in LDS, prefix, scatter (the order inside an expert's run depends on the
@@ -101,8 +130,8 @@ extern "C" int hymeta_moe_route_sigmoid(const hymeta_moe_route_sigmoid_args* arg
     return HYMETA_ERR_INVALID_ARG;
   hipStream_t st = begin_launches(stream);
   if (a.num_tokens > 0) {
-    if (a.act_dtype == HYMETA_BF16) hipLaunchKernelGGL(moe_scores_topk_kernel<ActBf16>, dim3(a.num_tokens), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL(moe_scores_topk_kernel<ActF32>, dim3(a.num_tokens), dim3(256), 0, st, a);
+    if (a.act_dtype == HYMETA_BF16) hipLaunchKernelGGL(moe_scores_topk_kernel<ActBf16>, dim3((a.num_tokens + kRouteTokens - 1) / kRouteTokens), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(moe_scores_topk_kernel<ActF32>, dim3((a.num_tokens + kRouteTokens - 1) / kRouteTokens), dim3(256), 0, st, a);
   }
   hipLaunchKernelGGL(moe_sort_pairs_kernel, dim3(1), dim3(kSortThreads), 0, st, a);
   return launch_status();

@@ -22,11 +22,25 @@ __global__ __launch_bounds__(256) void token_shift_kernel(hymeta_token_shift_arg
   const float* prev = first ? nullptr : x - a.x_stride_t;
   float* st = (slot >= 0 && a.state != nullptr) ? a.state + static_cast<int64_t>(slot) * a.width : nullptr;
   const float* last = a.x + static_cast<int64_t>(r1 - 1) * a.x_stride_t;
-  for (int c = threadIdx.x; c < a.width; c += 256) {
-    const float h = x[c];
-    const float hp = first ? (from_state ? st[c] : 0.f) : prev[c];
-    A::st(out + c, h + (hp - h) * a.mix[c]);
-    if (first && st != nullptr) st[c] = last[c];
+  // four columns a round: their loads are in flight together (a short row is one round trip to memory, not four)
+  for (int c0 = threadIdx.x; c0 < a.width; c0 += 4 * 256) {
+    float h[4], hp[4], mx[4], lt[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = c0 + 256 * u;
+      const bool ok = c < a.width;
+      h[u] = ok ? x[c] : 0.f;
+      hp[u] = ok ? (first ? (from_state ? st[c] : 0.f) : prev[c]) : 0.f;
+      mx[u] = ok ? a.mix[c] : 0.f;
+      lt[u] = (ok && first && st != nullptr) ? last[c] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int c = c0 + 256 * u;
+      if (c >= a.width) continue;
+      A::st(out + c, h[u] + (hp[u] - h[u]) * mx[u]);
+      if (first && st != nullptr) st[c] = lt[u];
+    }
   }
 }
 
@@ -38,8 +52,35 @@ __device__ __forceinline__ float summed(const hymeta_add_group_norm_args& a, con
   return z;
 }
 
-// grid = rows; the groups one after the other, each with a sum over the workgroup.
+// grid = rows; the groups one after the other, each with a sum over the workgroup.  Rows of up to kNormCached columns
+// are read once: a thread keeps its columns of the sum in registers between the statistics and the scaling.
+constexpr int kNormPerThread = 16, kNormCached = 256 * kNormPerThread;
+
 template <typename A>
+__device__ __forceinline__ void load4(const typename A::elem* p, float* v);
+template <>
+__device__ __forceinline__ void load4<ActF32>(const float* p, float* v) {
+  const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+  v[0] = t[0], v[1] = t[1], v[2] = t[2], v[3] = t[3];
+}
+template <>
+__device__ __forceinline__ void load4<ActBf16>(const uint16_t* p, float* v) {
+  const u32x2 t = *reinterpret_cast<const u32x2*>(p);
+  v[0] = lo_bf(t[0]), v[1] = hi_bf(t[0]), v[2] = lo_bf(t[1]), v[3] = hi_bf(t[1]);
+}
+template <typename A>
+__device__ __forceinline__ void store4(typename A::elem* p, const float* v);
+template <>
+__device__ __forceinline__ void store4<ActF32>(float* p, const float* v) { *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]}; }
+template <>
+__device__ __forceinline__ void store4<ActBf16>(uint16_t* p, const float* v) {
+  *reinterpret_cast<u32x2*>(p) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+}
+
+// Mode 0: any shape, two passes over the row.  Mode 1: rows of up to kNormCached columns, read once, a thread keeps its
+// columns between the statistics and the scaling.  Mode 2: the same with four consecutive columns per load and store
+// (groups, strides and pointers in whole fours).
+template <typename A, int Mode>
 __global__ __launch_bounds__(256) void add_group_norm_kernel(hymeta_add_group_norm_args a) {
   typedef typename A::elem elem;
   __shared__ float red[4];
@@ -50,21 +91,90 @@ __global__ __launch_bounds__(256) void add_group_norm_kernel(hymeta_add_group_no
   const elem* y2 = a.y2 ? static_cast<const elem*>(a.y2) + t * a.y2_stride_t : nullptr;
   elem* out = a.out ? static_cast<elem*>(a.out) + t * a.width : nullptr;
   const int part = a.width / a.groups;
+  float z[Mode ? kNormPerThread : 1];
+  // column of this thread's value u
+  auto col = [&](int u) { return Mode == 2 ? 4 * (static_cast<int>(threadIdx.x) + 256 * (u >> 2)) + (u & 3) : static_cast<int>(threadIdx.x) + 256 * u; };
+  if (Mode == 1) {
+#pragma unroll
+    for (int u = 0; u < kNormPerThread; ++u) z[u] = col(u) < a.width ? summed(a, x, y, y2, col(u), bf) : 0.f;
+  }
+  if (Mode == 2) {
+#pragma unroll
+    for (int u = 0; u < kNormPerThread; u += 4) {
+      const int c = col(u);
+      float xv[4] = {}, yv[4] = {}, y2v[4] = {};
+      if (c < a.width) {
+        load4<ActF32>(x + c, xv);
+        if (y) load4<A>(y + c, yv);
+        if (y2) load4<A>(y2 + c, y2v);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float s = a.alpha * xv[e];
+        if (y) s += yv[e];
+        if (y2) s += y2v[e];
+        z[u + e] = s;
+      }
+    }
+  }
   for (int g = 0; g < a.groups; ++g) {
     const int lo = g * part;
     float ss = 0.f;
-    for (int c = lo + threadIdx.x; c < lo + part; c += 256) {
-      const float z = summed(a, x, y, y2, c, bf);
-      ss = fmaf(z, z, ss);
+    if (Mode) {
+#pragma unroll
+      for (int u = 0; u < kNormPerThread; ++u)
+        if (col(u) >= lo && col(u) < lo + part) ss = fmaf(z[u], z[u], ss);
+    } else {
+      for (int c = lo + threadIdx.x; c < lo + part; c += 256) {
+        const float v = summed(a, x, y, y2, c, bf);
+        ss = fmaf(v, v, ss);
+      }
     }
     ss = block_sum<4>(ss, red);
     const float inv = 1.f / sqrtf(ss / static_cast<float>(part) + a.eps);
-    for (int c = lo + threadIdx.x; c < lo + part; c += 256) {
-      const float v = summed(a, x, y, y2, c, bf) * inv * a.weight[c];
-      if (out) A::st(out + c, v);
-      if (a.in_place) x[c] = v;
+    if (Mode == 2) {
+#pragma unroll
+      for (int u = 0; u < kNormPerThread; u += 4) {
+        const int c = col(u);
+        if (c >= lo && c < lo + part) {
+          float wv[4], v[4];
+          load4<ActF32>(a.weight + c, wv);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = z[u + e] * inv * wv[e];
+          if (out) store4<A>(out + c, v);
+          if (a.in_place) store4<ActF32>(x + c, v);
+        }
+      }
+    } else if (Mode == 1) {
+#pragma unroll
+      for (int u = 0; u < kNormPerThread; ++u) {
+        const int c = col(u);
+        if (c >= lo && c < lo + part) {
+          const float v = z[u] * inv * a.weight[c];
+          if (out) A::st(out + c, v);
+          if (a.in_place) x[c] = v;
+        }
+      }
+    } else {
+      for (int c = lo + threadIdx.x; c < lo + part; c += 256) {
+        const float v = summed(a, x, y, y2, c, bf) * inv * a.weight[c];
+        if (out) A::st(out + c, v);
+        if (a.in_place) x[c] = v;
+      }
     }
   }
+}
+
+template <typename A>
+void launch_add_group_norm(const hymeta_add_group_norm_args& a, hipStream_t st) {
+  const int elem = A::kDtype == HYMETA_BF16 ? 2 : 4;
+  auto whole4 = [&](const void* p, int64_t stride, int bytes) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) % (4 * bytes) == 0 && stride % 4 == 0); };
+  const bool fours = (a.width / a.groups) % 4 == 0 && whole4(a.x, a.x_stride_t, 4) && whole4(a.y, a.y_stride_t, elem) &&
+                     whole4(a.y2, a.y2_stride_t, elem) && whole4(a.out, 0, elem) && whole4(a.weight, 0, 4);
+  const dim3 grid(a.num_tokens), block(256);
+  if (a.width > kNormCached) hipLaunchKernelGGL((add_group_norm_kernel<A, 0>), grid, block, 0, st, a);
+  else if (fours) hipLaunchKernelGGL((add_group_norm_kernel<A, 2>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((add_group_norm_kernel<A, 1>), grid, block, 0, st, a);
 }
 
 }  // namespace
@@ -96,7 +206,7 @@ extern "C" int hymeta_add_group_norm(const hymeta_add_group_norm_args* args, hym
   if (!a.x || !a.weight || a.x_stride_t < a.width || (!a.out && !a.in_place)) return HYMETA_ERR_INVALID_ARG;
   if ((a.y && a.y_stride_t < a.width) || (a.y2 && a.y2_stride_t < a.width)) return HYMETA_ERR_INVALID_ARG;
   hipStream_t st = begin_launches(stream);
-  if (a.act_dtype == HYMETA_BF16) hipLaunchKernelGGL(add_group_norm_kernel<ActBf16>, dim3(a.num_tokens), dim3(256), 0, st, a);
-  else hipLaunchKernelGGL(add_group_norm_kernel<ActF32>, dim3(a.num_tokens), dim3(256), 0, st, a);
+  if (a.act_dtype == HYMETA_BF16) launch_add_group_norm<ActBf16>(a, st);
+  else launch_add_group_norm<ActF32>(a, st);
   return launch_status();
 }

@@ -473,6 +473,12 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void sink_attention_prefill_mfm
 // maximum and denominator, rows padded to whole 16 bytes.
 __host__ __device__ inline size_t partial_row_floats(int dv) { return static_cast<size_t>(dv) + 4; }
 constexpr int kDecodeWaves = 4;
+// Whether the four waves of a decode workgroup merge their partials in LDS (the two tile images, free after the last
+// tile, hold them) and write one partial per slice: a quarter of the partials' traffic and of the combine's work.
+template <int D, int DV, int RB>
+struct DecodeMerge {
+  static constexpr bool value = 2 * sizeof(MfmaSmem<D, DV>) >= sizeof(float) * kDecodeWaves * 16 * RB * (DV + 4);
+};
 
 // Decode: a workgroup per (sequence with one row, key/value head, slice of the keys); rows = the group's query heads; the
 // four waves share the staged tiles and take a 16-key subtile each.  Every wave writes its (maximum, denominator,
@@ -490,8 +496,10 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
   const int j_hi = min(pos, j_lo + tiles_per_split * kTileKeys - 1);
   int first = 0;
   if (a.window_left >= 0) first = max(0, pos - a.window_left);
+  constexpr bool kMerge = DecodeMerge<D, DV, RB>::value;
   float* part = static_cast<float*>(a.workspace) +
-                (((static_cast<size_t>(s) * a.num_kv_heads + g) * splits + split) * kDecodeWaves + wave) * (HG * partial_row_floats(DV));
+                (((static_cast<size_t>(s) * a.num_kv_heads + g) * splits + split) * (kMerge ? 1 : kDecodeWaves) + (kMerge ? 0 : wave)) *
+                    (HG * partial_row_floats(DV));
   const int32_t* bt = a.block_tables + static_cast<int64_t>(s) * a.block_table_stride;
   WaveRows<D, DV, RB> w;
 #pragma unroll
@@ -526,6 +534,8 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
     }
     __syncthreads();
   }
+  constexpr int kRowF = DV + 4;
+  float* lds = reinterpret_cast<float*>(&sm[0]);            // (the loop ended on a barrier: nobody reads the tiles any more)
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     float l = w.l[rb];
@@ -533,17 +543,41 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
     l += __shfl_xor(l, 32, 64);
     const int r = 16 * rb + n;
     if (r >= HG) continue;
-    float* pr = part + r * partial_row_floats(DV);
+    float* pr = kMerge ? lds + (wave * 16 * RB + r) * kRowF : part + r * partial_row_floats(DV);
     if (g4 == 0) pr[DV] = w.m[rb], pr[DV + 1] = l;
 #pragma unroll
     for (int cb = 0; cb < DV / 16; ++cb)
       *reinterpret_cast<f32x4v*>(pr + 16 * cb + 4 * g4) = w.o[rb][cb];
   }
+  if constexpr (kMerge) {
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < HG * (DV / 4); idx += 64 * kDecodeWaves) {
+      const int r = idx / (DV / 4), c4 = idx % (DV / 4);
+      float mw[kDecodeWaves], m = -INFINITY;
+#pragma unroll
+      for (int v = 0; v < kDecodeWaves; ++v) {
+        mw[v] = lds[(v * 16 * RB + r) * kRowF + DV];
+        m = fmaxf(m, mw[v]);
+      }
+      f32x4v o = f32x4v{0.f, 0.f, 0.f, 0.f};
+      float l = 0.f;
+#pragma unroll
+      for (int v = 0; v < kDecodeWaves; ++v) {
+        if (mw[v] == -INFINITY) continue;                   // a wave that saw no key of this row
+        const float f = __builtin_amdgcn_exp2f(mw[v] - m);
+        o += *reinterpret_cast<const f32x4v*>(lds + (v * 16 * RB + r) * kRowF + 4 * c4) * f;
+        l += lds[(v * 16 * RB + r) * kRowF + DV + 1] * f;
+      }
+      float* pr = part + r * partial_row_floats(DV);
+      *reinterpret_cast<f32x4v*>(pr + 4 * c4) = o;
+      if (c4 == 0) pr[DV] = m, pr[DV + 1] = l;
+    }
+  }
 }
 
 // grid = (sequences, heads), 64 threads: merge the slices of a decode row, add the sink, normalise, store bf16.
 __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymeta_sink_attention_args a, int splits) {
-  splits *= kDecodeWaves;                // every wave of a slice wrote a partial of its own
+  // (splits: partials per (sequence, key/value head): one per slice, or one per wave of a slice)
   const int s = blockIdx.x, h = blockIdx.y;
   const int t = a.query_start_loc[s];
   if (a.query_start_loc[s + 1] - t != 1) return;
@@ -602,11 +636,15 @@ int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st) {
   const int tiles = (a.max_seq_len + kTileKeys - 1) / kTileKeys;
   const int tiles_per_split = (tiles + splits - 1) / splits;
   const dim3 grid(splits, a.num_kv_heads, a.num_seqs);
-  if (a.num_heads / a.num_kv_heads <= 16)
+  int parts;
+  if (a.num_heads / a.num_kv_heads <= 16) {
     hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 1, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split);
-  else
+    parts = splits * (DecodeMerge<D, DV, 1>::value ? 1 : kDecodeWaves);
+  } else {
     hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 2, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split);
-  hipLaunchKernelGGL(sink_attention_decode_combine_kernel, dim3(a.num_seqs, a.num_heads), dim3(64), 0, st, a, splits);
+    parts = splits * (DecodeMerge<D, DV, 2>::value ? 1 : kDecodeWaves);
+  }
+  hipLaunchKernelGGL(sink_attention_decode_combine_kernel, dim3(a.num_seqs, a.num_heads), dim3(64), 0, st, a, parts);
   return launch_status();
 }
 
