@@ -12,6 +12,14 @@ struct ActBf16 {
   static __device__ __forceinline__ float ld(const elem* p) { return bf2f(*p); }
   static __device__ __forceinline__ void st(elem* p, float v) { *p = f2bf(v); }
   static __device__ __forceinline__ float round(float v) { return bf16_round(v); }
+  // four consecutive elements, 8-byte aligned
+  static __device__ __forceinline__ void ld4(const elem* p, float* v) {
+    const u32x2 t = *reinterpret_cast<const u32x2*>(p);
+    v[0] = lo_bf(t[0]), v[1] = hi_bf(t[0]), v[2] = lo_bf(t[1]), v[3] = hi_bf(t[1]);
+  }
+  static __device__ __forceinline__ void st4(elem* p, const float* v) {
+    *reinterpret_cast<u32x2*>(p) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+  }
   // fp32 in, fp32 out, the hardware's exponential (about 2 ulp): where the inputs carry 8 bits
   static __device__ __forceinline__ float sigmoid(float x) { return 1.f / (1.f + __expf(-x)); }
 };
@@ -22,6 +30,12 @@ struct ActF32 {
   static __device__ __forceinline__ float ld(const elem* p) { return *p; }
   static __device__ __forceinline__ void st(elem* p, float v) { *p = v; }
   static __device__ __forceinline__ float round(float v) { return v; }
+  // four consecutive elements, 16-byte aligned
+  static __device__ __forceinline__ void ld4(const elem* p, float* v) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+    v[0] = t[0], v[1] = t[1], v[2] = t[2], v[3] = t[3];
+  }
+  static __device__ __forceinline__ void st4(elem* p, const float* v) { *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]}; }
   static __device__ __forceinline__ float sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
 };
 

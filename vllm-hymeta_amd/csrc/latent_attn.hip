@@ -9,14 +9,18 @@ namespace {
 
 constexpr int kMaxRotPairs = 256;
 
-// cos and sin of position * freq, times mag, for the pairs that turn; (1, 0) for the pairs that pass unchanged.
+// cos and sin of position * freq, times mag, for the pairs that turn; (1, 0) for the pairs that pass unchanged.  The
+// angle is formed and brought into [-pi, pi] in double precision (a position of a million times a frequency near one
+// keeps all its digits); the functions themselves are the fp32 ones on that remainder.
 __device__ __forceinline__ void fill_rotation(float* s_cos, float* s_sin, const double* freqs, int pairs, int turning, int pos, float mag) {
+  constexpr double kTwoPi = 6.283185307179586476925286766559, kInvTwoPi = 0.15915494309189533576888376337251;
   for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
     float c = 1.f, s = 0.f;
     if (i < turning) {
       const double ang = static_cast<double>(pos) * freqs[i];
-      c = static_cast<float>(cos(ang) * static_cast<double>(mag));
-      s = static_cast<float>(sin(ang) * static_cast<double>(mag));
+      const float r = static_cast<float>(fma(-kTwoPi, rint(ang * kInvTwoPi), ang));
+      c = cosf(r) * mag;
+      s = sinf(r) * mag;
     }
     s_cos[i] = c;
     s_sin[i] = s;
@@ -77,12 +81,16 @@ __global__ __launch_bounds__(256) void latent_q_assemble_kernel(hymeta_latent_q_
   __syncthreads();
   const elem* q = static_cast<const elem*>(a.q) + static_cast<int64_t>(t) * a.q_stride_t;
   elem* out = static_cast<elem*>(a.out) + static_cast<int64_t>(t) * a.num_heads * (C + a.rot_dim);
-  for (int h = 0; h < a.num_heads; ++h) {
-    const elem* qa = static_cast<const elem*>(a.q_abs) + (static_cast<int64_t>(h) * a.num_tokens + t) * C;
+  // one element of the absorbed part, or one pair of the rotated part, per thread and round, over all heads at once
+  const int per_head = C + pairs;
+  for (int idx = threadIdx.x; idx < a.num_heads * per_head; idx += 256) {
+    const int h = idx / per_head, j = idx % per_head;
     elem* o = out + static_cast<int64_t>(h) * (C + a.rot_dim);
-    for (int c = threadIdx.x; c < C; c += 256) o[c] = qa[c];
-    const elem* qr = q + static_cast<int64_t>(h) * (a.dim + a.rot_dim) + a.dim;
-    for (int i = threadIdx.x; i < pairs; i += 256) {
+    if (j < C) {
+      o[j] = static_cast<const elem*>(a.q_abs)[(static_cast<int64_t>(h) * a.num_tokens + t) * C + j];
+    } else {
+      const int i = j - C;
+      const elem* qr = q + static_cast<int64_t>(h) * (a.dim + a.rot_dim) + a.dim;
       const float u = A::ld(qr + 2 * i), v = A::ld(qr + 2 * i + 1);
       A::st(o + C + 2 * i, u * s_cos[i] - v * s_sin[i]);
       A::st(o + C + 2 * i + 1, v * s_cos[i] + u * s_sin[i]);

@@ -56,27 +56,6 @@ __device__ __forceinline__ float summed(const hymeta_add_group_norm_args& a, con
 // are read once: a thread keeps its columns of the sum in registers between the statistics and the scaling.
 constexpr int kNormPerThread = 16, kNormCached = 256 * kNormPerThread;
 
-template <typename A>
-__device__ __forceinline__ void load4(const typename A::elem* p, float* v);
-template <>
-__device__ __forceinline__ void load4<ActF32>(const float* p, float* v) {
-  const f32x4 t = *reinterpret_cast<const f32x4*>(p);
-  v[0] = t[0], v[1] = t[1], v[2] = t[2], v[3] = t[3];
-}
-template <>
-__device__ __forceinline__ void load4<ActBf16>(const uint16_t* p, float* v) {
-  const u32x2 t = *reinterpret_cast<const u32x2*>(p);
-  v[0] = lo_bf(t[0]), v[1] = hi_bf(t[0]), v[2] = lo_bf(t[1]), v[3] = hi_bf(t[1]);
-}
-template <typename A>
-__device__ __forceinline__ void store4(typename A::elem* p, const float* v);
-template <>
-__device__ __forceinline__ void store4<ActF32>(float* p, const float* v) { *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]}; }
-template <>
-__device__ __forceinline__ void store4<ActBf16>(uint16_t* p, const float* v) {
-  *reinterpret_cast<u32x2*>(p) = u32x2{pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-}
-
 // Mode 0: any shape, two passes over the row.  Mode 1: rows of up to kNormCached columns, read once, a thread keeps its
 // columns between the statistics and the scaling.  Mode 2: the same with four consecutive columns per load and store
 // (groups, strides and pointers in whole fours).
@@ -104,9 +83,9 @@ __global__ __launch_bounds__(256) void add_group_norm_kernel(hymeta_add_group_no
       const int c = col(u);
       float xv[4] = {}, yv[4] = {}, y2v[4] = {};
       if (c < a.width) {
-        load4<ActF32>(x + c, xv);
-        if (y) load4<A>(y + c, yv);
-        if (y2) load4<A>(y2 + c, y2v);
+        ActF32::ld4(x + c, xv);
+        if (y) A::ld4(y + c, yv);
+        if (y2) A::ld4(y2 + c, y2v);
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -138,11 +117,11 @@ __global__ __launch_bounds__(256) void add_group_norm_kernel(hymeta_add_group_no
         const int c = col(u);
         if (c >= lo && c < lo + part) {
           float wv[4], v[4];
-          load4<ActF32>(a.weight + c, wv);
+          ActF32::ld4(a.weight + c, wv);
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = z[u + e] * inv * wv[e];
-          if (out) store4<A>(out + c, v);
-          if (a.in_place) store4<ActF32>(x + c, v);
+          if (out) A::st4(out + c, v);
+          if (a.in_place) ActF32::st4(x + c, v);
         }
       }
     } else if (Mode == 1) {
