@@ -42,7 +42,7 @@ def test_config_reads_every_size_and_the_layers_that_share_weights():
         GeponexConfig(chain)
 
 
-@pytest.mark.parametrize("dims,base,scaling", [(32, 500000.0, {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}),
+@pytest.mark.parametrize("dims,base,scaling", [(24, 300000.0, {"factor": 6.0, "original": 2048, "fast": 24.0, "slow": 2.0}),
                                                (8, 10000.0, {"factor": 4.0, "original": 64, "fast": 16.0, "slow": 2.0}),
                                                (64, 10000.0, {"factor": 40.0, "original": 4096, "fast": 32.0, "slow": 1.0}),
                                                (16, 1000000.0, None)])

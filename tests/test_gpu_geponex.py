@@ -241,7 +241,7 @@ _YARN = {"factor": 4.0, "original": 64, "fast": 16.0, "slow": 2.0}
 @pytest.mark.parametrize("kind,mixer", [
     ("latent_attention_2", latent_mixer_config()),
     ("latent_attention", latent_mixer_config(scaling=_YARN)),
-    ("latent_attention", latent_mixer_config(heads=4, dim=32, rot_dim=32, vdim=32, kv_rank=64, q_rank=80, base=500000.0, scaling=_YARN)),
+    ("latent_attention", latent_mixer_config(heads=5, dim=16, rot_dim=32, vdim=48, kv_rank=64, q_rank=72, base=300000.0, scaling=_YARN)),
     ("latent_attention_2", latent_mixer_config(heads=1, dim=8, rot_dim=16, vdim=8, kv_rank=24, q_rank=16)),
 ])
 def test_latent_attention_sublayer_in_portions(dtype, kind, mixer):
@@ -450,9 +450,9 @@ MODELS = {
         ("latent_attention", latent_mixer_config(heads=1, dim=8, rot_dim=4, vdim=8, kv_rank=12, q_rank=10), moe_config(experts=3, top=1, ff=24, shared_ff=0)),
         ("latent_attention_2", latent_mixer_config(heads=2, dim=8, rot_dim=8, vdim=4, kv_rank=20, q_rank=16), _DENSE)]),
     "matrix_core_sizes": dict(width=128, groups=2, alpha=2.0, layers=[
-        ("latent_attention_2", latent_mixer_config(heads=8, dim=32, rot_dim=32, vdim=32, kv_rank=64, q_rank=96), {"kind": "dense", "ff": 192}),
+        ("latent_attention_2", latent_mixer_config(heads=6, dim=16, rot_dim=32, vdim=48, kv_rank=64, q_rank=96), {"kind": "dense", "ff": 192}),
         ("lightning", lightning_mixer_config(heads=2, dim=32, vdim=64, decay=[0.7, 0.995]), moe_config(experts=8, top=2, ff=64, shared_ff=64)),
-        ("latent_attention", latent_mixer_config(heads=4, dim=64, rot_dim=64, vdim=64, kv_rank=128, q_rank=64, base=500000.0, scaling=_YARN),
+        ("latent_attention", latent_mixer_config(heads=3, dim=64, rot_dim=64, vdim=32, kv_rank=128, q_rank=64, base=200000.0, scaling=_YARN),
          moe_config(experts=8, top=2, ff=64, shared_ff=64)),
         ("weights_of", 1), ("weights_of", 0)]),
     "lightning_first_weights_shared_twice": dict(width=64, groups=4, alpha=0.5, layers=[
@@ -587,3 +587,51 @@ def test_long_decode_keeps_its_states():
     eng.finish_request("d")
     got = eng.run_batch([("x", toks[:201], [200])])
     assert rel_err(got, ref) < 5e-5
+
+
+def test_trace_runner_and_generate_command_lines(tmp_path):
+    """A checkpoint folder (config.json + model.safetensors) served by the two programs under bin/: the trace replayer
+    runs portions, single tokens and two requests side by side, gives pages back at a request's end and writes the logits
+    asked for (fp32 against the oracle); the generator's greedy tokens are the oracle's argmax."""
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    from safetensors.torch import save_file
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = geponex_config(**MODELS["default"])
+    weights = {k: v.to(torch.bfloat16).float() for k, v in geponex_random_weights(cfg, seed=12).items()}      # what a bf16 file holds
+    model_dir = tmp_path / "model"
+    model_dir.mkdir()
+    (model_dir / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in weights.items()}, str(model_dir / "model.safetensors"))
+    a, b = _tokens(90, cfg["vocab"], 5), _tokens(40, cfg["vocab"], 6)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:50], "want": [0, 49]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[50:52], "want": []}, {"id": "b", "tokens": b[:39], "want": [38]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[39:], "want": [0]}, {"id": "a", "tokens": a[52:53], "want": [0]}], "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[53:], "want": [36]}, {"id": "c", "tokens": b[:7], "want": [6]}], "end": ["a", "c"]},
+    ]
+    out_dir = tmp_path / "out"
+    run = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(model_dir), "--dtype", "float32", "--out", str(out_dir),
+                          "--max-tokens", "192"], input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert [l for l in run.stdout.splitlines() if l.startswith("done")] == [f"done {k}" for k in range(4)]
+    ra, rb = geponex_ref(cfg, weights, a), geponex_ref(cfg, weights, b)
+    want = {0: torch.stack([ra[0], ra[49]]), 1: rb[38:39], 2: torch.stack([rb[39], ra[52]]), 3: torch.stack([ra[89], rb[6]])}
+    for k, ref in want.items():
+        got = torch.from_numpy(np.fromfile(str(out_dir / f"{k}.f32"), dtype="<f4").reshape(ref.shape[0], -1))
+        assert rel_err(got, ref) < 5e-5, k
+    gen = subprocess.run([sys.executable, os.path.join(root, "bin", "generate"), "--model", str(model_dir), "--dtype", "float32", "--prompt-ids",
+                          ",".join(map(str, a[:20])), "--max-new-tokens", "3", "--max-tokens", "128"], capture_output=True, text=True, timeout=300)
+    assert gen.returncode == 0, gen.stderr[-2000:]
+    line = json.loads([l for l in gen.stdout.splitlines() if l.startswith("{")][-1])
+    toks = list(a[:20])
+    for t in line["output"]:
+        logits = geponex_ref(cfg, weights, toks)[-1]
+        top2 = logits.topk(2).values
+        if float(top2[0] - top2[1]) > 1e-3:
+            assert t == int(logits.argmax())
+        toks.append(t)
+    assert len(line["output"]) == 3
