@@ -473,11 +473,19 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void sink_attention_prefill_mfm
 // maximum and denominator, rows padded to whole 16 bytes.
 __host__ __device__ inline size_t partial_row_floats(int dv) { return static_cast<size_t>(dv) + 4; }
 constexpr int kDecodeWaves = 4;
-// Whether the four waves of a decode workgroup merge their partials in LDS (the two tile images, free after the last
-// tile, hold them) and write one partial per slice: a quarter of the partials' traffic and of the combine's work.
+// LDS images of a decode workgroup: two (the next tile goes into the other image while this one is multiplied) where
+// both fit in 72 KB, which leaves two workgroups on a compute unit; one for larger tiles, so that three or four
+// workgroups overlap each other instead.
+template <int D, int DV>
+struct DecodeImages {
+  static constexpr int value = 2 * sizeof(MfmaSmem<D, DV>) <= 72 * 1024 ? 2 : 1;
+};
+// Whether the four waves of a decode workgroup merge their partials through LDS (the tile images, free after the last
+// tile, hold two waves' rows at a time: waves 2, 3 hand theirs to waves 0, 1, then wave 1 to wave 0) and write one
+// partial per slice: a quarter of the partials' traffic and of the combine's work.
 template <int D, int DV, int RB>
 struct DecodeMerge {
-  static constexpr bool value = 2 * sizeof(MfmaSmem<D, DV>) >= sizeof(float) * kDecodeWaves * 16 * RB * (DV + 4);
+  static constexpr bool value = DecodeImages<D, DV>::value * sizeof(MfmaSmem<D, DV>) >= sizeof(float) * 2 * 16 * RB * (DV + 4);
 };
 
 // Decode: a workgroup per (sequence with one row, key/value head, slice of the keys); rows = the group's query heads; the
@@ -485,7 +493,8 @@ struct DecodeMerge {
 // weighted values) per head; the combine kernel merges them and the sink.
 template <int D, int DV, int RB, bool VinK>
 __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_kernel(hymeta_sink_attention_args a, int splits, int tiles_per_split) {
-  __shared__ MfmaSmem<D, DV> sm[2];
+  constexpr int kImages = DecodeImages<D, DV>::value;
+  __shared__ MfmaSmem<D, DV> sm[kImages];
   const int s = blockIdx.z, g = blockIdx.y, split = blockIdx.x;
   const int t = a.query_start_loc[s];
   if (a.query_start_loc[s + 1] - t != 1) return;
@@ -521,57 +530,87 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
   if (j_lo <= j_hi) {
     stage.issue(a, bt, g, j_lo, j_hi);
     stage.commit(sm[0]);
-    if (j_lo + kTileKeys <= j_hi) stage.issue(a, bt, g, j_lo + kTileKeys, j_hi);
+    if (kImages == 2 && j_lo + kTileKeys <= j_hi) stage.issue(a, bt, g, j_lo + kTileKeys, j_hi);
   }
   __syncthreads();
-  int buf = 0;
-  for (int j0 = j_lo; j0 <= j_hi; j0 += kTileKeys, buf ^= 1) {
-    if (j0 + kTileKeys <= j_hi) stage.commit(sm[buf ^ 1]);
-    if (j0 + 2 * kTileKeys <= j_hi) stage.issue(a, bt, g, j0 + 2 * kTileKeys, j_hi);
-    if (j0 + 16 * wave <= j_hi) {
-      if (a.window_left < 0 && j0 + kTileKeys - 1 <= pos) attend_tile<D, DV, RB, 1, false>(w, sm[buf], a, j0, wave);
-      else attend_tile<D, DV, RB, 1, true>(w, sm[buf], a, j0, wave);
+  if constexpr (kImages == 2) {
+    int buf = 0;
+    for (int j0 = j_lo; j0 <= j_hi; j0 += kTileKeys, buf ^= 1) {
+      if (j0 + kTileKeys <= j_hi) stage.commit(sm[buf ^ 1]);
+      if (j0 + 2 * kTileKeys <= j_hi) stage.issue(a, bt, g, j0 + 2 * kTileKeys, j_hi);
+      if (j0 + 16 * wave <= j_hi) {
+        if (a.window_left < 0 && j0 + kTileKeys - 1 <= pos) attend_tile<D, DV, RB, 1, false>(w, sm[buf], a, j0, wave);
+        else attend_tile<D, DV, RB, 1, true>(w, sm[buf], a, j0, wave);
+      }
+      __syncthreads();
     }
-    __syncthreads();
+  } else {
+    // one image: the next tile's loads are in flight while this one is multiplied and go into LDS behind a barrier
+    for (int j0 = j_lo; j0 <= j_hi; j0 += kTileKeys) {
+      const bool more = j0 + kTileKeys <= j_hi;
+      if (more) stage.issue(a, bt, g, j0 + kTileKeys, j_hi);
+      if (j0 + 16 * wave <= j_hi) {
+        if (a.window_left < 0 && j0 + kTileKeys - 1 <= pos) attend_tile<D, DV, RB, 1, false>(w, sm[0], a, j0, wave);
+        else attend_tile<D, DV, RB, 1, true>(w, sm[0], a, j0, wave);
+      }
+      __syncthreads();
+      if (more) {
+        stage.commit(sm[0]);
+        __syncthreads();
+      }
+    }
   }
   constexpr int kRowF = DV + 4;
   float* lds = reinterpret_cast<float*>(&sm[0]);            // (the loop ended on a barrier: nobody reads the tiles any more)
+  float lr[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     float l = w.l[rb];
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
-    const int r = 16 * rb + n;
-    if (r >= HG) continue;
-    float* pr = kMerge ? lds + (wave * 16 * RB + r) * kRowF : part + r * partial_row_floats(DV);
-    if (g4 == 0) pr[DV] = w.m[rb], pr[DV + 1] = l;
-#pragma unroll
-    for (int cb = 0; cb < DV / 16; ++cb)
-      *reinterpret_cast<f32x4v*>(pr + 16 * cb + 4 * g4) = w.o[rb][cb];
+    lr[rb] = l;
   }
-  if constexpr (kMerge) {
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < HG * (DV / 4); idx += 64 * kDecodeWaves) {
-      const int r = idx / (DV / 4), c4 = idx % (DV / 4);
-      float mw[kDecodeWaves], m = -INFINITY;
+  // this wave's rows into LDS place `slot`, or (to == part) into the workspace
+  auto put = [&](float* to, int rows_limit) {
 #pragma unroll
-      for (int v = 0; v < kDecodeWaves; ++v) {
-        mw[v] = lds[(v * 16 * RB + r) * kRowF + DV];
-        m = fmaxf(m, mw[v]);
-      }
-      f32x4v o = f32x4v{0.f, 0.f, 0.f, 0.f};
-      float l = 0.f;
+    for (int rb = 0; rb < RB; ++rb) {
+      const int r = 16 * rb + n;
+      if (r >= rows_limit) continue;
+      float* pr = to + r * kRowF;
+      if (g4 == 0) pr[DV] = w.m[rb], pr[DV + 1] = lr[rb];
 #pragma unroll
-      for (int v = 0; v < kDecodeWaves; ++v) {
-        if (mw[v] == -INFINITY) continue;                   // a wave that saw no key of this row
-        const float f = __builtin_amdgcn_exp2f(mw[v] - m);
-        o += *reinterpret_cast<const f32x4v*>(lds + (v * 16 * RB + r) * kRowF + 4 * c4) * f;
-        l += lds[(v * 16 * RB + r) * kRowF + DV + 1] * f;
-      }
-      float* pr = part + r * partial_row_floats(DV);
-      *reinterpret_cast<f32x4v*>(pr + 4 * c4) = o;
-      if (c4 == 0) pr[DV] = m, pr[DV + 1] = l;
+      for (int cb = 0; cb < DV / 16; ++cb) *reinterpret_cast<f32x4v*>(pr + 16 * cb + 4 * g4) = w.o[rb][cb];
     }
+  };
+  // another wave's rows from LDS merged into this wave's
+  auto take = [&](const float* from) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const float* pr = from + (16 * rb + n) * kRowF;
+      const float mp = pr[DV], lp = pr[DV + 1];
+      const float m = fmaxf(w.m[rb], mp);
+      const float f = w.m[rb] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w.m[rb] - m);      // (a wave that saw no key of the row)
+      const float fp = mp == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mp - m);
+#pragma unroll
+      for (int cb = 0; cb < DV / 16; ++cb) w.o[rb][cb] = w.o[rb][cb] * f + *reinterpret_cast<const f32x4v*>(pr + 16 * cb + 4 * g4) * fp;
+      lr[rb] = lr[rb] * f + lp * fp;
+      w.m[rb] = m;
+    }
+  };
+  if constexpr (kMerge) {
+    static_assert(kDecodeWaves == 4, "the merge is a tree over four waves");
+    if (wave >= 2) put(lds + (wave - 2) * 16 * RB * kRowF, 16 * RB);
+    __syncthreads();
+    if (wave < 2) take(lds + wave * 16 * RB * kRowF);
+    __syncthreads();
+    if (wave == 1) put(lds, 16 * RB);
+    __syncthreads();
+    if (wave == 0) {
+      take(lds);
+      put(part, HG);
+    }
+  } else {
+    put(part, HG);
   }
 }
 
@@ -617,9 +656,14 @@ inline bool mfma_shape(const hymeta_sink_attention_args& a) {
          (reinterpret_cast<uintptr_t>(a.q) | reinterpret_cast<uintptr_t>(a.kv_cache) | reinterpret_cast<uintptr_t>(a.out)) % 16 == 0;
 }
 
-inline int decode_splits(int num_seqs, int num_kv_heads, int max_seq_len) {
+inline int decode_splits(int num_seqs, int num_heads, int num_kv_heads, int max_seq_len) {
   const int tiles = (max_seq_len + kTileKeys - 1) / kTileKeys;
-  int splits = (1024 + num_seqs * num_kv_heads - 1) / (num_seqs * num_kv_heads);     // about four workgroups per compute unit
+  // Workgroups aimed at: a workgroup's fixed cost (query fragments, first tile, the merge of its waves, its partial) grows
+  // with the query heads it carries, so fewer, longer workgroups pay.  Measured at 64 sequences x 4096 keys: 28 heads on
+  // one row of 192: 93 / 67 / 56 / 87 us at 1024 / 512 / 256 / 128; 16 heads on it: 53 / 40 / 45; 4 key/value heads with
+  // 7 query heads each: 125 / 114 / 168.
+  const int target = num_heads / num_kv_heads > 16 ? 256 : 512;
+  int splits = (target + num_seqs * num_kv_heads - 1) / (num_seqs * num_kv_heads);
   splits = splits < 1 ? 1 : splits;
   return splits > tiles ? (tiles < 1 ? 1 : tiles) : splits;
 }
@@ -632,7 +676,7 @@ int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st) {
     hipLaunchKernelGGL((sink_attention_prefill_mfma_kernel<D, DV, kRB, VinK>), grid, dim3(64 * kPrefillWaves), 0, st, a);
   }
   // sequences with a single row: every step but a pure prompt step has some; a prompt of one token is one too
-  const int splits = decode_splits(a.num_seqs, a.num_kv_heads, a.max_seq_len);
+  const int splits = decode_splits(a.num_seqs, a.num_heads, a.num_kv_heads, a.max_seq_len);
   const int tiles = (a.max_seq_len + kTileKeys - 1) / kTileKeys;
   const int tiles_per_split = (tiles + splits - 1) / splits;
   const dim3 grid(splits, a.num_kv_heads, a.num_seqs);
@@ -674,7 +718,7 @@ extern "C" int hymeta_qk_norm_cache(const hymeta_qk_norm_cache_args* args, hymet
 extern "C" size_t hymeta_sink_attention_workspace_bytes(int32_t num_seqs, int32_t num_heads, int32_t num_kv_heads, int32_t v_dim,
                                                         int32_t max_seq_len) {
   if (num_seqs <= 0 || num_heads <= 0 || num_kv_heads <= 0 || v_dim <= 0) return 0;
-  const int splits = decode_splits(num_seqs, num_kv_heads, max_seq_len < 1 ? 1 : max_seq_len);
+  const int splits = decode_splits(num_seqs, num_heads, num_kv_heads, max_seq_len < 1 ? 1 : max_seq_len);
   return static_cast<size_t>(num_seqs) * splits * kDecodeWaves * num_heads * partial_row_floats(v_dim) * sizeof(float);
 }
 
