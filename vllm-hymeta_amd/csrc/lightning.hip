@@ -11,14 +11,14 @@ __device__ __forceinline__ float silu_f(float x) { return x / (1.f + expf(-x)); 
 // Token by token.  grid = (heads, sequences, value columns in runs of 256); a thread owns one value column c and keeps
 // that column of the state, S[:, c], in registers; q_t and k_t go through LDS.
 template <typename A, int DMAX>
-__global__ __launch_bounds__(256) void lightning_rows_kernel(hymeta_lightning_attention_args a, int max_rows) {
+__global__ __launch_bounds__(256) void lightning_rows_kernel(hymeta_lightning_attention_args a, int min_rows, int max_rows) {
   typedef typename A::elem elem;
   __shared__ float s_q[2][DMAX], s_k[2][DMAX];
   const int h = blockIdx.x, s = blockIdx.y;
   const int c = blockIdx.z * 256 + threadIdx.x;
   const int H = a.num_heads, D = a.head_dim, Dv = a.v_dim;
   const int r0 = a.query_start_loc[s], r1 = a.query_start_loc[s + 1];
-  if (r1 <= r0 || r1 - r0 > max_rows) return;          // longer portions: the chunked kernel's
+  if (r1 - r0 < min_rows || r1 - r0 > max_rows) return;          // single rows / longer portions: the other kernels'
   const int slot = a.slot_idx[s];
   const bool live = c < Dv;
   float* st = (slot >= 0) ? a.state + ((static_cast<int64_t>(slot) * H + h) * D) * Dv : nullptr;
@@ -311,14 +311,79 @@ inline bool chunk_shape(const hymeta_lightning_attention_args& a) {
          reinterpret_cast<uintptr_t>(a.out) % 16 == 0 && a.v_dim / kSliceV <= 65535;
 }
 
+// Sequences with one row (decode).  grid = (heads, sequences), 256 threads over the state in fours of value columns: a
+// thread takes the columns 4 c4 .. 4 c4 + 3 of the rows d0, d0 + dstep, ... of S (16-byte loads and stores, four rows in
+// flight together), the partial outputs of the dstep row groups meet in LDS.
+constexpr int kStepMaxD = 256;
 template <typename A>
-void launch_rows(const hymeta_lightning_attention_args& a, hipStream_t st, int max_rows) {
+__global__ __launch_bounds__(256) void lightning_step_kernel(hymeta_lightning_attention_args a) {
+  typedef typename A::elem elem;
+  __shared__ float s_q[kStepMaxD], s_k[kStepMaxD];
+  __shared__ __attribute__((aligned(16))) float s_o[256 * 4];
+  const int h = blockIdx.x, s = blockIdx.y;
+  const int t = a.query_start_loc[s];
+  if (a.query_start_loc[s + 1] - t != 1) return;
+  const int H = a.num_heads, D = a.head_dim, Dv = a.v_dim, Dv4 = Dv / 4;
+  const int c4 = threadIdx.x % Dv4, d0 = threadIdx.x / Dv4, dstep = 256 / Dv4;
+  const int slot = a.slot_idx[s];
+  float* st = slot >= 0 ? a.state + ((static_cast<int64_t>(slot) * H + h) * D) * Dv : nullptr;
+  const bool carry = st != nullptr && a.context_lens[s] > 0;
+  const elem* row = static_cast<const elem*>(a.qkv) + static_cast<int64_t>(t) * a.qkv_stride_t;
+  for (int d = threadIdx.x; d < D; d += 256) {
+    s_q[d] = silu_f(A::ld(row + static_cast<int64_t>(h) * D + d));
+    s_k[d] = silu_f(A::ld(row + static_cast<int64_t>(H + h) * D + d));
+  }
+  float v[4];
+  A::ld4(row + 2 * static_cast<int64_t>(H) * D + static_cast<int64_t>(h) * Dv + 4 * c4, v);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = silu_f(v[e]);
+  const float decay = a.decay[h];
+  __syncthreads();
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int db = d0; db < D; db += 4 * dstep) {
+    f32x4 S[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int d = db + u * dstep;
+      S[u] = (carry && d < D) ? *reinterpret_cast<const f32x4*>(st + static_cast<int64_t>(d) * Dv + 4 * c4) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int d = db + u * dstep;
+      if (d >= D) continue;
+      const float k = s_k[d], q = s_q[d];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        S[u][e] = fmaf(decay, S[u][e], k * v[e]);
+        acc[e] = fmaf(S[u][e], q, acc[e]);
+      }
+      if (st != nullptr) *reinterpret_cast<f32x4*>(st + static_cast<int64_t>(d) * Dv + 4 * c4) = S[u];
+    }
+  }
+  *reinterpret_cast<f32x4*>(&s_o[threadIdx.x * 4]) = acc;          // [d0][4 c4 + e]
+  __syncthreads();
+  for (int c = threadIdx.x; c < Dv; c += 256) {
+    float o = 0.f;
+    for (int g = 0; g < dstep; ++g) o += s_o[(g * Dv4 + c / 4) * 4 + (c & 3)];
+    a.out[static_cast<int64_t>(t) * H * Dv + static_cast<int64_t>(h) * Dv + c] = o;
+  }
+}
+
+inline bool step_shape(const hymeta_lightning_attention_args& a) {
+  const int dv4 = a.v_dim / 4;
+  const int bytes = a.act_dtype == HYMETA_BF16 ? 2 : 4;
+  return a.v_dim % 4 == 0 && dv4 <= 256 && 256 % dv4 == 0 && a.head_dim <= kStepMaxD && reinterpret_cast<uintptr_t>(a.state) % 16 == 0 &&
+         reinterpret_cast<uintptr_t>(a.qkv) % (4 * bytes) == 0 && a.qkv_stride_t % 4 == 0 && (2 * a.num_heads * a.head_dim) % 4 == 0;
+}
+
+template <typename A>
+void launch_rows(const hymeta_lightning_attention_args& a, hipStream_t st, int min_rows, int max_rows) {
   const dim3 grid(a.num_heads, a.num_seqs, (a.v_dim + 255) / 256);
   const dim3 block(a.v_dim >= 256 ? 256 : (a.v_dim + 63) / 64 * 64);
-  if (a.head_dim <= 32) hipLaunchKernelGGL((lightning_rows_kernel<A, 32>), grid, block, 0, st, a, max_rows);
-  else if (a.head_dim <= 64) hipLaunchKernelGGL((lightning_rows_kernel<A, 64>), grid, block, 0, st, a, max_rows);
-  else if (a.head_dim <= 128) hipLaunchKernelGGL((lightning_rows_kernel<A, 128>), grid, block, 0, st, a, max_rows);
-  else hipLaunchKernelGGL((lightning_rows_kernel<A, 256>), grid, block, 0, st, a, max_rows);
+  if (a.head_dim <= 32) hipLaunchKernelGGL((lightning_rows_kernel<A, 32>), grid, block, 0, st, a, min_rows, max_rows);
+  else if (a.head_dim <= 64) hipLaunchKernelGGL((lightning_rows_kernel<A, 64>), grid, block, 0, st, a, min_rows, max_rows);
+  else if (a.head_dim <= 128) hipLaunchKernelGGL((lightning_rows_kernel<A, 128>), grid, block, 0, st, a, min_rows, max_rows);
+  else hipLaunchKernelGGL((lightning_rows_kernel<A, 256>), grid, block, 0, st, a, min_rows, max_rows);
 }
 
 }  // namespace
@@ -345,8 +410,17 @@ extern "C" int hymeta_lightning_attention(const hymeta_lightning_attention_args*
     else hipLaunchKernelGGL(lightning_chunk_kernel<128>, grid, dim3(256), 0, st, a, kChunkMinRows);
     max_rows = kChunkMinRows - 1;
   }
-  if (a.act_dtype == HYMETA_BF16) launch_rows<ActBf16>(a, st, max_rows);
-  else launch_rows<ActF32>(a, st, max_rows);
+  int min_rows = 1;
+  if (step_shape(a)) {
+    const dim3 grid(a.num_heads, a.num_seqs);
+    if (a.act_dtype == HYMETA_BF16) hipLaunchKernelGGL(lightning_step_kernel<ActBf16>, grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(lightning_step_kernel<ActF32>, grid, dim3(256), 0, st, a);
+    min_rows = 2;
+  }
+  if (a.max_query_len >= min_rows && max_rows >= min_rows) {
+    if (a.act_dtype == HYMETA_BF16) launch_rows<ActBf16>(a, st, min_rows, max_rows);
+    else launch_rows<ActF32>(a, st, min_rows, max_rows);
+  }
   return launch_status();
 }
 
