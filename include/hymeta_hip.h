@@ -1349,9 +1349,14 @@ typedef struct hymeta_lightning_attention_args {
   const int32_t* query_start_loc;
   const int32_t* context_lens;
   const int32_t* slot_idx;
-  int32_t num_tokens, num_seqs, num_heads, head_dim, v_dim, act_dtype, max_query_len;
+  int32_t num_tokens, num_seqs, num_heads, head_dim, v_dim, act_dtype, max_query_len;   /* max_query_len: upper bound of the portions' rows */
   int64_t qkv_stride_t;
+  void* workspace;             /* hymeta_lightning_attention_workspace_bytes(...) bytes, or NULL when that is 0 */
+  size_t workspace_bytes;
 } hymeta_lightning_attention_args;
+/* > 0 for steps with long portions: they run in segments side by side (summarise / chain / apply: three launches). */
+size_t hymeta_lightning_attention_workspace_bytes(int32_t num_seqs, int32_t num_heads, int32_t head_dim, int32_t v_dim,
+                                                  int32_t max_query_len);
 int hymeta_lightning_attention(const hymeta_lightning_attention_args* args, hymeta_stream_t stream);
 
 /* out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * weight * sigmoid(gate[t]): the output norm and gate of a linear attention. */

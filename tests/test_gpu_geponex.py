@@ -332,6 +332,32 @@ def test_lightning_attention_prefill_equals_token_by_token_and_portions(dtype, m
             assert rel_err(state[2], s_whole) < (1e-5 if dtype == torch.float32 else 1e-2)
 
 
+def test_lightning_long_portions_run_in_segments():
+    """A portion of 2300 rows (segments of 1024 side by side, chained through their states) behind 70 rows that left a
+    state, beside a short portion and a decoding sequence in the same step: outputs and final states as token by token."""
+    mixer = lightning_mixer_config(heads=2, dim=32, vdim=64, decay=[0.97, 0.9995])
+    W, eps, T = 32, 1e-6, 2370
+    cfg = geponex_config(width=W, layers=[("lightning", mixer, None)])
+    weights = geponex_random_weights(cfg, seed=11)
+    w = {k[len("l0.mix."):]: v.double() for k, v in weights.items() if k.startswith("l0.mix.")}
+    g = torch.Generator().manual_seed(12)
+    h, h2, h3 = bf16_values(T, W, gen=g), bf16_values(90, W, gen=g), bf16_values(31, W, gen=g)
+    ref, ref2, ref3 = lightning_ref(h, w, mixer, eps), lightning_ref(h2, w, mixer, eps), lightning_ref(h3, w, mixer, eps)
+    mod = _lightning_mixer(mixer, w, torch.bfloat16, eps)
+    state = torch.full((4, 2, 32, 64), 3.0, device=DEV)
+    dev = lambda t: t.to(torch.bfloat16).to(DEV)
+    first = mod(torch.cat([dev(h[:70]), dev(h3[:30])]), layout_of([70, 30], [0, 0], [1, 3]), state)
+    step = mod(torch.cat([dev(h[70:]), dev(h2), dev(h3[30:])]), layout_of([T - 70, 90, 1], [70, 0, 30], [1, 0, 3]), state)
+    assert rel_err(first[:70], ref[:70]) < 2e-2
+    assert rel_err(step[:T - 70], ref[70:]) < 2e-2 and rel_err(step[T - 70:T - 70 + 90], ref2) < 2e-2 and rel_err(step[-1:], ref3[30:]) < 2e-2
+    # the final states against a token-by-token run of the same rows
+    state2 = torch.zeros_like(state)
+    for t in range(T):
+        mod(dev(h[t:t + 1]), layout_of([1], [t], [2]), state2)
+    assert rel_err(state[1], state2[2]) < 2e-3
+    assert torch.all(state[2] == 3.0)
+
+
 def test_lightning_attention_batches_unequal_sequences():
     mixer = lightning_mixer_config(heads=2, dim=32, vdim=64, decay=[0.8, 0.99])
     W, eps = 64, 1e-6

@@ -104,6 +104,12 @@ __global__ __launch_bounds__(256) void gated_rms_norm_kernel(hymeta_gated_rms_no
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 constexpr int kChunk = HYMETA_LIGHTNING_CHUNK, kSliceV = 32;
 constexpr int kChunkMinRows = 8;            // shorter portions go token by token
+// Steps with a portion of kSegmentMinRows or more are cut into segments of kSegmentRows that run side by side: every
+// segment but the last is summarised from a zero state, the summaries are chained into the states in front of the
+// segments, then every segment runs from its state (three launches; a sequence's chunks otherwise follow each other in
+// one workgroup per head and value slice, which leaves most of the chip idle under a single long prompt).
+constexpr int kSegmentRows = 1024, kSegmentMinRows = 2048;
+enum ChunkMode { kWhole = 0, kSummarise = 1, kApply = 2 };
 
 __device__ __forceinline__ f32x4v mfma16(bf16x8 a, bf16x8 b, f32x4v c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
 
@@ -127,15 +133,21 @@ __device__ __forceinline__ u32x4 silu8(u32x4 raw, float* vals) {
 }
 
 template <int D>
-__global__ __launch_bounds__(256) void lightning_chunk_kernel(hymeta_lightning_attention_args a, int min_rows) {
+__global__ __launch_bounds__(256) void lightning_chunk_kernel(hymeta_lightning_attention_args a, int min_rows, int seg_rows, int nseg, int mode) {
   constexpr int PK = D + 8, PT = kChunk + 8, NBW = (2 * D / 16) / 4;
   __shared__ __attribute__((aligned(16))) uint16_t sk[kChunk * PK];          // silu(k), a row per key
   __shared__ __attribute__((aligned(16))) uint16_t skt[2][D * PT];           // decayed keys, transposed [d][key], hi / lo
   __shared__ __attribute__((aligned(16))) uint16_t svt[kSliceV * PT];        // silu(v) of the slice, transposed [c][key]
   __shared__ __attribute__((aligned(16))) uint16_t sst[2][kSliceV * PK];     // state^T [c][d], hi / lo
-  const int h = blockIdx.x, s = blockIdx.y, vs = blockIdx.z;
-  const int r0 = a.query_start_loc[s], rows = a.query_start_loc[s + 1] - r0;
-  if (rows < min_rows) return;
+  const int h = blockIdx.x, s = blockIdx.y / nseg, seg = blockIdx.y % nseg, vs = blockIdx.z;
+  const int r0 = a.query_start_loc[s], rows_all = a.query_start_loc[s + 1] - r0;
+  if (rows_all < min_rows) return;
+  // this workgroup's rows of the portion: all of them (kWhole), or one segment
+  const int r_lo = mode == kWhole ? 0 : seg * seg_rows;
+  if (r_lo >= rows_all) return;
+  const int rows = mode == kWhole ? rows_all : min(rows_all, r_lo + seg_rows);        // (end of the rows, not their count)
+  const bool last = rows == rows_all;
+  if (mode == kSummarise && last) return;                    // nothing comes behind the last segment
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, n = lane & 15, g4 = lane >> 4;
   const int H = a.num_heads, Dv = a.v_dim;
   const int slot = a.slot_idx[s];
@@ -143,11 +155,15 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(hymeta_lightning_a
   const float decay = a.decay[h];
   const float l2 = decay > 0.f ? log2f(decay) : -INFINITY;
   const bool carry = st != nullptr && a.context_lens[s] > 0;
+  // a segment's place in the workspace: its summary (kSummarise writes it), then the state in front of it (kApply reads it)
+  float* wsp = mode == kWhole ? nullptr
+                              : static_cast<float*>(a.workspace) + (((static_cast<int64_t>(s) * nseg + seg) * H + h) * D) * Dv + vs * kSliceV;
+  const float* init = mode == kWhole ? (carry ? st : nullptr) : mode == kApply ? wsp : nullptr;
   f32x4v S[NBW];
 #pragma unroll
   for (int ib = 0; ib < NBW; ++ib) {
     const int b = wave + 4 * ib, cb = b & 1, db = b >> 1;
-    S[ib] = carry ? *reinterpret_cast<const f32x4v*>(st + static_cast<int64_t>(16 * db + n) * Dv + 16 * cb + 4 * g4) : f32x4v{0.f, 0.f, 0.f, 0.f};
+    S[ib] = init ? *reinterpret_cast<const f32x4v*>(init + static_cast<int64_t>(16 * db + n) * Dv + 16 * cb + 4 * g4) : f32x4v{0.f, 0.f, 0.f, 0.f};
   }
   auto state_to_lds = [&]() {
 #pragma unroll
@@ -189,12 +205,12 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(hymeta_lightning_a
 #pragma unroll
     for (int sd = 0; sd < D / 32; ++sd) {
       rq[sd] = u32x4{0u, 0u, 0u, 0u};
-      if (i < nrow) rq[sd] = ld16g(base + i * a.qkv_stride_t + q_off + 32 * sd + 8 * g4);
+      if (i < nrow && mode != kSummarise) rq[sd] = ld16g(base + i * a.qkv_stride_t + q_off + 32 * sd + 8 * g4);
     }
   };
   static_assert(kChunk * (kSliceV / 8) == 256, "one group of the value slice per thread");
-  fetch(0);
-  for (int c0 = 0; c0 < rows; c0 += kChunk) {
+  fetch(r_lo);
+  for (int c0 = r_lo; c0 < rows; c0 += kChunk) {
     const int nrow = min(kChunk, rows - c0);
     const uint16_t* base = qkv + static_cast<int64_t>(r0 + c0) * a.qkv_stride_t;
     (void)base;
@@ -227,57 +243,59 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(hymeta_lightning_a
     for (int sd = 0; sd < D / 32; ++sd) q[sd] = __builtin_bit_cast(bf16x8, silu8(rq[sd], nullptr));
     __syncthreads();
     if (c0 + kChunk < rows) fetch(c0 + kChunk);        // in flight while this chunk is multiplied
-    // weights of the chunk's own rows: (q_i . k_j) L^(i-j) for j <= i, as hi + lo parts
-    uint32_t phi[4][2], plo[4][2];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      f32x4v sc = f32x4v{0.f, 0.f, 0.f, 0.f};
-      if (ks <= wave) {
-#pragma unroll
-        for (int sd = 0; sd < D / 32; ++sd)
-          sc = mfma16(__builtin_bit_cast(bf16x8, ld16(&sk[(16 * ks + n) * PK + 32 * sd + 8 * g4])), q[sd], sc);
+    if (mode != kSummarise) {
+      // weights of the chunk's own rows: (q_i . k_j) L^(i-j) for j <= i, as hi + lo parts
+      uint32_t phi[4][2], plo[4][2];
+  #pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        f32x4v sc = f32x4v{0.f, 0.f, 0.f, 0.f};
+        if (ks <= wave) {
+  #pragma unroll
+          for (int sd = 0; sd < D / 32; ++sd)
+            sc = mfma16(__builtin_bit_cast(bf16x8, ld16(&sk[(16 * ks + n) * PK + 32 * sd + 8 * g4])), q[sd], sc);
+        }
+        float p[4];
+  #pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int j = 16 * ks + 4 * g4 + r;
+          p[r] = (ks <= wave && j <= i) ? sc[r] * decay_pow(l2, i - j) : 0.f;
+        }
+  #pragma unroll
+        for (int r2 = 0; r2 < 2; ++r2) {
+          const uint32_t hi = pack_bf16x2(p[2 * r2], p[2 * r2 + 1]);
+          phi[ks][r2] = hi;
+          plo[ks][r2] = pack_bf16x2(p[2 * r2] - lo_bf(hi), p[2 * r2 + 1] - hi_bf(hi));
+        }
       }
-      float p[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int j = 16 * ks + 4 * g4 + r;
-        p[r] = (ks <= wave && j <= i) ? sc[r] * decay_pow(l2, i - j) : 0.f;
+      f32x4v o[2];
+      const float row_decay = decay_pow(l2, i + 1);
+  #pragma unroll
+      for (int cb = 0; cb < 2; ++cb) {
+        // the state before the chunk
+        f32x4v x = f32x4v{0.f, 0.f, 0.f, 0.f};
+  #pragma unroll
+        for (int sd = 0; sd < D / 32; ++sd) {
+          x = mfma16(__builtin_bit_cast(bf16x8, ld16(&sst[0][(16 * cb + n) * PK + 32 * sd + 8 * g4])), q[sd], x);
+          x = mfma16(__builtin_bit_cast(bf16x8, ld16(&sst[1][(16 * cb + n) * PK + 32 * sd + 8 * g4])), q[sd], x);
+        }
+        f32x4v acc = x * row_decay;
+  #pragma unroll
+        for (int kp = 0; kp < 2; ++kp) {
+          if (2 * kp > wave) continue;
+          // k index 8 g4 + e of the product: keys 32 kp + 4 g4 + e for e < 4, 32 kp + 16 + 4 g4 + e - 4 after
+          const u32x2 v0 = *reinterpret_cast<const u32x2*>(&svt[(16 * cb + n) * PT + 32 * kp + 4 * g4]);
+          const u32x2 v1 = *reinterpret_cast<const u32x2*>(&svt[(16 * cb + n) * PT + 32 * kp + 16 + 4 * g4]);
+          const bf16x8 vf = __builtin_bit_cast(bf16x8, (u32x4{v0[0], v0[1], v1[0], v1[1]}));
+          acc = mfma16(vf, __builtin_bit_cast(bf16x8, (u32x4{phi[2 * kp][0], phi[2 * kp][1], phi[2 * kp + 1][0], phi[2 * kp + 1][1]})), acc);
+          acc = mfma16(vf, __builtin_bit_cast(bf16x8, (u32x4{plo[2 * kp][0], plo[2 * kp][1], plo[2 * kp + 1][0], plo[2 * kp + 1][1]})), acc);
+        }
+        o[cb] = acc;
       }
-#pragma unroll
-      for (int r2 = 0; r2 < 2; ++r2) {
-        const uint32_t hi = pack_bf16x2(p[2 * r2], p[2 * r2 + 1]);
-        phi[ks][r2] = hi;
-        plo[ks][r2] = pack_bf16x2(p[2 * r2] - lo_bf(hi), p[2 * r2 + 1] - hi_bf(hi));
+      if (i < nrow) {
+        float* orow = a.out + static_cast<int64_t>(r0 + c0 + i) * H * Dv + static_cast<int64_t>(h) * Dv + vs * kSliceV;
+  #pragma unroll
+        for (int cb = 0; cb < 2; ++cb) *reinterpret_cast<f32x4v*>(orow + 16 * cb + 4 * g4) = o[cb];
       }
-    }
-    f32x4v o[2];
-    const float row_decay = decay_pow(l2, i + 1);
-#pragma unroll
-    for (int cb = 0; cb < 2; ++cb) {
-      // the state before the chunk
-      f32x4v x = f32x4v{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int sd = 0; sd < D / 32; ++sd) {
-        x = mfma16(__builtin_bit_cast(bf16x8, ld16(&sst[0][(16 * cb + n) * PK + 32 * sd + 8 * g4])), q[sd], x);
-        x = mfma16(__builtin_bit_cast(bf16x8, ld16(&sst[1][(16 * cb + n) * PK + 32 * sd + 8 * g4])), q[sd], x);
-      }
-      f32x4v acc = x * row_decay;
-#pragma unroll
-      for (int kp = 0; kp < 2; ++kp) {
-        if (2 * kp > wave) continue;
-        // k index 8 g4 + e of the product: keys 32 kp + 4 g4 + e for e < 4, 32 kp + 16 + 4 g4 + e - 4 after
-        const u32x2 v0 = *reinterpret_cast<const u32x2*>(&svt[(16 * cb + n) * PT + 32 * kp + 4 * g4]);
-        const u32x2 v1 = *reinterpret_cast<const u32x2*>(&svt[(16 * cb + n) * PT + 32 * kp + 16 + 4 * g4]);
-        const bf16x8 vf = __builtin_bit_cast(bf16x8, (u32x4{v0[0], v0[1], v1[0], v1[1]}));
-        acc = mfma16(vf, __builtin_bit_cast(bf16x8, (u32x4{phi[2 * kp][0], phi[2 * kp][1], phi[2 * kp + 1][0], phi[2 * kp + 1][1]})), acc);
-        acc = mfma16(vf, __builtin_bit_cast(bf16x8, (u32x4{plo[2 * kp][0], plo[2 * kp][1], plo[2 * kp + 1][0], plo[2 * kp + 1][1]})), acc);
-      }
-      o[cb] = acc;
-    }
-    if (i < nrow) {
-      float* orow = a.out + static_cast<int64_t>(r0 + c0 + i) * H * Dv + static_cast<int64_t>(h) * Dv + vs * kSliceV;
-#pragma unroll
-      for (int cb = 0; cb < 2; ++cb) *reinterpret_cast<f32x4v*>(orow + 16 * cb + 4 * g4) = o[cb];
     }
     // the state after the chunk
     const float chunk_decay = decay_pow(l2, nrow);
@@ -296,12 +314,36 @@ __global__ __launch_bounds__(256) void lightning_chunk_kernel(hymeta_lightning_a
     __syncthreads();            // every wave is done with this chunk's tiles and with the old state's image
     state_to_lds();             // (made visible by the barrier after the next chunk's staging)
   }
-  if (st != nullptr) {
+  float* to = mode == kSummarise ? wsp : (last ? st : nullptr);
+  if (to != nullptr) {
 #pragma unroll
     for (int ib = 0; ib < NBW; ++ib) {
       const int b = wave + 4 * ib, cb = b & 1, db = b >> 1;
-      *reinterpret_cast<f32x4v*>(st + static_cast<int64_t>(16 * db + n) * Dv + 16 * cb + 4 * g4) = S[ib];
+      *reinterpret_cast<f32x4v*>(to + static_cast<int64_t>(16 * db + n) * Dv + 16 * cb + 4 * g4) = S[ib];
     }
+  }
+}
+
+// The segments' summaries (each segment's state had it started from zero) become the states in front of the segments:
+// run = carried state; per segment: place <- run, run <- decay^(segment's rows) run + summary.  An element per thread.
+__global__ __launch_bounds__(256) void lightning_chain_kernel(hymeta_lightning_attention_args a, int min_rows, int seg_rows, int nseg) {
+  const int s = blockIdx.y;
+  const int rows = a.query_start_loc[s + 1] - a.query_start_loc[s];
+  if (rows < min_rows) return;
+  const int64_t per_head = static_cast<int64_t>(a.head_dim) * a.v_dim, per_seq = per_head * a.num_heads;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= per_seq) return;
+  const int h = static_cast<int>(idx / per_head);
+  const float decay = a.decay[h];
+  const float l2 = decay > 0.f ? log2f(decay) : -INFINITY;
+  const int slot = a.slot_idx[s];
+  float run = (slot >= 0 && a.context_lens[s] > 0) ? a.state[static_cast<int64_t>(slot) * per_seq + idx] : 0.f;
+  const int segs = (rows + seg_rows - 1) / seg_rows;
+  float* p = static_cast<float*>(a.workspace) + static_cast<int64_t>(s) * nseg * per_seq + idx;
+  for (int seg = 0; seg < segs; ++seg, p += per_seq) {
+    const float summary = seg < segs - 1 ? *p : 0.f;
+    *p = run;
+    run = decay_pow(l2, min(seg_rows, rows - seg * seg_rows)) * run + summary;
   }
 }
 
@@ -392,6 +434,13 @@ void launch_rows(const hymeta_lightning_attention_args& a, hipStream_t st, int m
 
 using namespace hymeta;
 
+extern "C" size_t hymeta_lightning_attention_workspace_bytes(int32_t num_seqs, int32_t num_heads, int32_t head_dim, int32_t v_dim,
+                                                             int32_t max_query_len) {
+  if (num_seqs <= 0 || num_heads <= 0 || head_dim <= 0 || v_dim <= 0 || max_query_len < kSegmentMinRows) return 0;
+  const size_t nseg = (static_cast<size_t>(max_query_len) + kSegmentRows - 1) / kSegmentRows;
+  return nseg * num_seqs * num_heads * head_dim * v_dim * sizeof(float);
+}
+
 extern "C" int hymeta_lightning_attention(const hymeta_lightning_attention_args* args, hymeta_stream_t stream) {
   if (!args_ok(args)) return HYMETA_ERR_INVALID_ARG;
   const hymeta_lightning_attention_args& a = *args;
@@ -404,10 +453,25 @@ extern "C" int hymeta_lightning_attention(const hymeta_lightning_attention_args*
   hipStream_t st = begin_launches(stream);
   int max_rows = 0x7fffffff;
   if (chunk_shape(a) && a.max_query_len >= kChunkMinRows) {
-    const dim3 grid(a.num_heads, a.num_seqs, a.v_dim / kSliceV);
-    if (a.head_dim == 32) hipLaunchKernelGGL(lightning_chunk_kernel<32>, grid, dim3(256), 0, st, a, kChunkMinRows);
-    else if (a.head_dim == 64) hipLaunchKernelGGL(lightning_chunk_kernel<64>, grid, dim3(256), 0, st, a, kChunkMinRows);
-    else hipLaunchKernelGGL(lightning_chunk_kernel<128>, grid, dim3(256), 0, st, a, kChunkMinRows);
+    const size_t need = hymeta_lightning_attention_workspace_bytes(a.num_seqs, a.num_heads, a.head_dim, a.v_dim, a.max_query_len);
+    const int nseg = need > 0 ? (a.max_query_len + kSegmentRows - 1) / kSegmentRows : 1;
+    if (need > 0 && (!a.workspace || a.workspace_bytes < need)) return HYMETA_ERR_WORKSPACE;
+    if (static_cast<int64_t>(a.num_seqs) * nseg > 65535) return HYMETA_ERR_UNSUPPORTED;
+    const dim3 grid(a.num_heads, a.num_seqs * nseg, a.v_dim / kSliceV);
+    auto chunks = [&](int mode) {
+      if (a.head_dim == 32) hipLaunchKernelGGL(lightning_chunk_kernel<32>, grid, dim3(256), 0, st, a, kChunkMinRows, kSegmentRows, nseg, mode);
+      else if (a.head_dim == 64) hipLaunchKernelGGL(lightning_chunk_kernel<64>, grid, dim3(256), 0, st, a, kChunkMinRows, kSegmentRows, nseg, mode);
+      else hipLaunchKernelGGL(lightning_chunk_kernel<128>, grid, dim3(256), 0, st, a, kChunkMinRows, kSegmentRows, nseg, mode);
+    };
+    if (nseg == 1) {
+      chunks(kWhole);
+    } else {
+      chunks(kSummarise);
+      const int64_t per_seq = static_cast<int64_t>(a.num_heads) * a.head_dim * a.v_dim;
+      hipLaunchKernelGGL(lightning_chain_kernel, dim3(static_cast<unsigned>((per_seq + 255) / 256), a.num_seqs), dim3(256), 0, st, a, kChunkMinRows,
+                         kSegmentRows, nseg);
+      chunks(kApply);
+    }
     max_rows = kChunkMinRows - 1;
   }
   int min_rows = 1;

@@ -440,7 +440,7 @@ class LightningAttentionArgs(_Args):
         ("query_start_loc", _ptr), ("context_lens", _ptr), ("slot_idx", _ptr),
         ("num_tokens", _i32), ("num_seqs", _i32), ("num_heads", _i32), ("head_dim", _i32), ("v_dim", _i32), ("act_dtype", _i32),
         ("max_query_len", _i32),
-        ("qkv_stride_t", _i64),
+        ("qkv_stride_t", _i64), ("workspace", _ptr), ("workspace_bytes", _sz),
     ]
 
 
@@ -557,6 +557,7 @@ _SIGNATURES = {
     "hymeta_add_group_norm": (C.c_int, [C.POINTER(AddGroupNormArgs), _ptr]),
     "hymeta_latent_kv_prep": (C.c_int, [C.POINTER(LatentKvPrepArgs), _ptr]),
     "hymeta_latent_q_assemble": (C.c_int, [C.POINTER(LatentQAssembleArgs), _ptr]),
+    "hymeta_lightning_attention_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32, _i32]),
     "hymeta_lightning_attention": (C.c_int, [C.POINTER(LightningAttentionArgs), _ptr]),
     "hymeta_gated_rms_norm": (C.c_int, [C.POINTER(GatedRmsNormArgs), _ptr]),
     "hymeta_activation": (C.c_int, [C.POINTER(ActivationArgs), _ptr]),

@@ -1856,7 +1856,12 @@ def lightning_attention(qkv: torch.Tensor, state: torch.Tensor, decay: torch.Ten
     a.query_start_loc, a.context_lens, a.slot_idx = _p(query_start_loc), _p(context_lens), _p(slot_idx)
     a.num_tokens, a.num_seqs, a.num_heads, a.head_dim, a.v_dim, a.act_dtype, a.max_query_len = T, S, H, D, Dv, _act(qkv), max_query_len
     a.qkv_stride_t = qkv.stride(0)
-    _C.check(_C.load().hymeta_lightning_attention(C.byref(a), _stream(qkv)), "hymeta_lightning_attention")
+    lib = _C.load()
+    nbytes = int(lib.hymeta_lightning_attention_workspace_bytes(S, H, D, Dv, max_query_len))
+    if nbytes:
+        ws = _workspace(qkv.device, nbytes, "lightning")
+        a.workspace, a.workspace_bytes = _p(ws), ws.numel()
+    _C.check(lib.hymeta_lightning_attention(C.byref(a), _stream(qkv)), "hymeta_lightning_attention")
     return out
 
 
