@@ -124,6 +124,17 @@ def kernel_table(dev, W, H, B, ctx, L, E, top, ff, C=128, R=64, D=128):
     qd2, kvd2 = rnd(B, H, D), rnd(B * bps, BLOCK, G, 2 * D)
     add(f"sink_attention decode (Sonuzen) B={B} ctx={ctx}",
         lambda: hip_ops.sink_attention(qd2, kvd2, btd, qsl, sl, G, D, D, D ** -0.5, 1, ctx + 1, r1, r2), nbytes=B * G * (ctx + 1) * 2 * D * 2)
+    # ---- a latent of 512 + 64 (value slices of 128, each launch repeats the scores), 16 heads
+    Cw, Hw = 512, 16
+    qw, kvw = rnd(L, Hw, Cw + R), rnd(nblk, BLOCK, 1, Cw + R)
+    sinkw = rnd(Hw, dtype=torch.float32)
+    add(f"latent attention prefill L={L} (H={Hw}, {Cw}+{R})",
+        lambda: hip_ops.sink_attention(qw, kvw, bt, i32([0, L]), i32([L]), 1, Cw + R, Cw, 0.05, L, L, sink=True, sink_logits=sinkw, value_in_key=True),
+        flops=Hw * L * L * (2 * Cw + R), iters=3)
+    qwd, kvwd = rnd(B, Hw, Cw + R), rnd(B * bps, BLOCK, 1, Cw + R)
+    add(f"latent attention decode B={B} ctx={ctx} (H={Hw}, {Cw}+{R})",
+        lambda: hip_ops.sink_attention(qwd, kvwd, btd, qsl, sl, 1, Cw + R, Cw, 0.05, 1, ctx + 1, sink=True, sink_logits=sinkw, value_in_key=True),
+        nbytes=B * (ctx + 1) * (Cw + R) * 2)
     # ---- the rest of the latent attention around its matrix products
     Q = W // 4
     proj = rnd(L, Q + C + R)

@@ -1179,7 +1179,8 @@ enum hymeta_bias_mode { HYMETA_BIAS_NONE = 0, HYMETA_BIAS_LOG_DISTANCE = 1 };
  * elements (hymeta_qk_norm_cache).  VALUE_IN_KEY: head_dim elements, of which the first v_dim are also the value (a
  * latent shared by keys and values followed by a rotated key part: hymeta_latent_kv_prep); v_dim <= head_dim.  With
  * VALUE_IN_KEY bf16 rows with v_dim 64 or 128 and head_dim = v_dim + 32 or v_dim + 64 run on the matrix cores (the
- * kernels of KEY_THEN_VALUE with another staging of the tiles); other sizes a wave per (row, head). */
+ * kernels of KEY_THEN_VALUE with another staging of the tiles), and so do v_dim 256 / 384 / 512 with head_dim = v_dim + 64,
+ * as 2 / 3 / 4 launches over value slices of 128; other sizes a wave per (row, head). */
 enum hymeta_kv_layout { HYMETA_KV_KEY_THEN_VALUE = 0, HYMETA_KV_VALUE_IN_KEY = 1 };
 typedef struct hymeta_sink_attention_args {
   uint32_t struct_size;

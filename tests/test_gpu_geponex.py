@@ -134,7 +134,8 @@ def _paged_rows(rows, dtype, block_size, shuffle_seed=0):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,C,R,sink", [(3, 40, 8, True), (4, 64, 32, False), (8, 128, 64, True), (1, 24, 0, True), (16, 64, 32, True)])
+@pytest.mark.parametrize("H,C,R,sink", [(3, 40, 8, True), (4, 64, 32, False), (8, 128, 64, True), (1, 24, 0, True), (16, 64, 32, True),
+                                       (4, 256, 64, True), (3, 384, 64, False), (20, 512, 64, True)])
 def test_attention_over_rows_shared_by_keys_and_values(dtype, H, C, R, sink):
     """Portions of a prompt and single rows over pages, against the plain statement; the sink logit of every head counts."""
     from vllm_hymeta import hip_ops
@@ -158,13 +159,14 @@ def test_attention_over_rows_shared_by_keys_and_values(dtype, H, C, R, sink):
     assert rel_err(torch.cat(outs), ref) < (2e-6 if dtype == torch.float32 else 1e-2)
 
 
+@pytest.mark.parametrize("C,R", [(64, 32), (512, 64)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_a_row_far_back_decides_the_output(dtype):
+def test_a_row_far_back_decides_the_output(dtype, C, R):
     """Among 700 rows one (at a page border, far from the query) matches the query's direction with a large score: the
     output is that row's value part, in a prompt's portion and for a single decoded row alike."""
     from vllm_hymeta import hip_ops
     g = torch.Generator().manual_seed(5)
-    T, H, C, R, bs = 700, 4, 64, 32, 64
+    T, H, bs = 700, 4, 64
     rows = bf16_values(T, C + R, std=0.3, gen=g)
     q = bf16_values(T, H, C + R, std=0.3, gen=g)
     far = 64                                            # first row of the second page

@@ -162,6 +162,12 @@ __device__ __forceinline__ f32x4v mfma16(bf16x8 a, bf16x8 b, f32x4v c) {
 constexpr int kTileKeys = 64;
 constexpr int kRowsPerWave = 32;
 
+// The value columns one launch computes: `first` .. `first` + DV of the `total` columns of a value row (and of an output
+// row).  Values wider than the kernels' DV run as several launches over slices (each repeats the scores).
+struct ValueSlice {
+  int first, total;
+};
+
 template <int D, int DV>
 struct MfmaSmem {
   static constexpr int kPitchK = D + 8;               // bf16 elements per key row (16-byte reads of 16 rows: no bank conflict)
@@ -187,6 +193,7 @@ struct TileStage {
   static_assert(D % 32 == 0 && DV % 16 == 0 && kValBlocks <= Threads && (!VinK || DV <= D), "the staging roles fit the workgroup");
   u32x4 rk[kKeyPerThread];
   u32x4 rv[4];
+  int value_at = kValueAt;      // where the staged value columns start in a head's part of a row
 
   // Pages hold a power of two of rows here (the host sends other sizes to the plain kernel).  A page of 64 rows or more
   // holds a whole tile (tiles start at multiples of 64): its number is one scalar load per tile, not a dependent vector
@@ -234,7 +241,7 @@ struct TileStage {
       for (int i = 0; i < 4; ++i) {
         const int j = j0 + 4 * grp + i;
         rv[i] = u32x4{0u, 0u, 0u, 0u};
-        if (j <= last) rv[i] = ld16g(row_ptr(p, j0, j) + kValueAt + ch * 8);
+        if (j <= last) rv[i] = ld16g(row_ptr(p, j0, j) + value_at + ch * 8);
       }
     }
   }
@@ -398,15 +405,20 @@ __device__ __forceinline__ void load_q(WaveRows<D, DV, RB>& w, int rb, const uin
     w.q[rb][st] = qrow ? __builtin_bit_cast(bf16x8, ld16g(qrow + 32 * st + 8 * g4)) : bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
 }
 
-constexpr int kPrefillWaves = 8;
-template <int RB> struct PrefillShape { static constexpr int kRows = 16 * RB * kPrefillWaves; };
+// Waves of a prompt workgroup: 8, or 4 for keys longer than 192 elements, whose query fragments (D / 8 registers) and
+// staging registers do not leave a wave of 8 its accumulators within 256 registers (408 bytes of scratch per lane at
+// 576; a workgroup of 4 waves has 512 registers per wave).
+template <int D> struct PrefillWaves { static constexpr int value = D > 192 ? 4 : 8; };
+template <int RB, int Waves> struct PrefillShape { static constexpr int kRows = 16 * RB * Waves; };
 
-// Portions of prompts: grid = (tiles of 128 RB rows, heads, sequences); a wave holds RB blocks of 16 rows; sequences with
+// Portions of prompts: grid = (tiles of 16 RB rows per wave, heads, sequences); a wave holds RB blocks of 16 rows; sequences with
 // one row are left to the decode form.
 template <int D, int DV, int RB, bool VinK>
-__global__ __launch_bounds__(64 * kPrefillWaves) void sink_attention_prefill_mfma_kernel(hymeta_sink_attention_args a) {
-  constexpr int kRows = PrefillShape<RB>::kRows;
-  __shared__ MfmaSmem<D, DV> sm[2];
+__global__ __launch_bounds__(64 * PrefillWaves<D>::value) void sink_attention_prefill_mfma_kernel(hymeta_sink_attention_args a, ValueSlice vs) {
+  constexpr int kPrefillWaves = PrefillWaves<D>::value;
+  constexpr int kRows = PrefillShape<RB, kPrefillWaves>::kRows;
+  constexpr int kImages = 2 * sizeof(MfmaSmem<D, DV>) <= 159 * 1024 ? 2 : 1;        // (160 KB of LDS)
+  __shared__ MfmaSmem<D, DV> sm[kImages];
   const int s = blockIdx.z, h = blockIdx.y;
   const int row0 = a.query_start_loc[s];
   const int q = a.query_start_loc[s + 1] - row0;
@@ -437,20 +449,39 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void sink_attention_prefill_mfm
   // two LDS images: while the waves multiply tile t out of one, tile t + 1 goes into the other and the loads of tile
   // t + 2 are in flight; one barrier per tile
   TileStage<D, DV, 64 * kPrefillWaves, VinK> stage;
+  if (VinK) stage.value_at = vs.first;
   stage.issue(a, bt, g, j_first, block_last);
   stage.commit(sm[0]);
-  if (j_first + kTileKeys <= block_last) stage.issue(a, bt, g, j_first + kTileKeys, block_last);
+  if (kImages == 2 && j_first + kTileKeys <= block_last) stage.issue(a, bt, g, j_first + kTileKeys, block_last);
   __syncthreads();
-  int buf = 0;
-  for (int j0 = j_first; j0 <= block_last; j0 += kTileKeys, buf ^= 1) {
-    if (j0 + kTileKeys <= block_last) stage.commit(sm[buf ^ 1]);
-    if (j0 + 2 * kTileKeys <= block_last) stage.issue(a, bt, g, j0 + 2 * kTileKeys, block_last);
-    if (wrow < q && j0 <= wave_last) {
-      // tiles wholly before the wave's first row (and no window) need no mask: every key is visible to every row
-      if (a.window_left < 0 && j0 + kTileKeys - 1 <= ctx + wrow) attend_tile<D, DV, RB, 4, false>(w, sm[buf], a, j0, 0);
-      else attend_tile<D, DV, RB, 4, true>(w, sm[buf], a, j0, 0);
+  if constexpr (kImages == 2) {
+    int buf = 0;
+    for (int j0 = j_first; j0 <= block_last; j0 += kTileKeys, buf ^= 1) {
+      if (j0 + kTileKeys <= block_last) stage.commit(sm[buf ^ 1]);
+      if (j0 + 2 * kTileKeys <= block_last) stage.issue(a, bt, g, j0 + 2 * kTileKeys, block_last);
+      if (wrow < q && j0 <= wave_last) {
+        // tiles wholly before the wave's first row (and no window) need no mask: every key is visible to every row
+        if (a.window_left < 0 && j0 + kTileKeys - 1 <= ctx + wrow) attend_tile<D, DV, RB, 4, false>(w, sm[buf], a, j0, 0);
+        else attend_tile<D, DV, RB, 4, true>(w, sm[buf], a, j0, 0);
+      }
+      __syncthreads();
     }
-    __syncthreads();
+  } else {
+    // one image (tiles of long rows): the next tile's loads are in flight while this one is multiplied and go into LDS
+    // behind a barrier
+    for (int j0 = j_first; j0 <= block_last; j0 += kTileKeys) {
+      const bool more = j0 + kTileKeys <= block_last;
+      if (more) stage.issue(a, bt, g, j0 + kTileKeys, block_last);
+      if (wrow < q && j0 <= wave_last) {
+        if (a.window_left < 0 && j0 + kTileKeys - 1 <= ctx + wrow) attend_tile<D, DV, RB, 4, false>(w, sm[0], a, j0, 0);
+        else attend_tile<D, DV, RB, 4, true>(w, sm[0], a, j0, 0);
+      }
+      __syncthreads();
+      if (more) {
+        stage.commit(sm[0]);
+        __syncthreads();
+      }
+    }
   }
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
@@ -460,7 +491,7 @@ __global__ __launch_bounds__(64 * kPrefillWaves) void sink_attention_prefill_mfm
     const int r = wrow + 16 * rb + n;
     if (r >= q) continue;
     const float inv = l > 0.f ? 1.f / l : 0.f;
-    uint16_t* out = static_cast<uint16_t*>(a.out) + (static_cast<int64_t>(row0 + r) * a.num_heads + h) * DV;
+    uint16_t* out = static_cast<uint16_t*>(a.out) + (static_cast<int64_t>(row0 + r) * a.num_heads + h) * vs.total + vs.first;
 #pragma unroll
     for (int cb = 0; cb < DV / 16; ++cb) {
       const f32x4v o = w.o[rb][cb] * inv;
@@ -492,7 +523,7 @@ struct DecodeMerge {
 // four waves share the staged tiles and take a 16-key subtile each.  Every wave writes its (maximum, denominator,
 // weighted values) per head; the combine kernel merges them and the sink.
 template <int D, int DV, int RB, bool VinK>
-__global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_kernel(hymeta_sink_attention_args a, int splits, int tiles_per_split) {
+__global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_kernel(hymeta_sink_attention_args a, int splits, int tiles_per_split, ValueSlice vs) {
   constexpr int kImages = DecodeImages<D, DV>::value;
   __shared__ MfmaSmem<D, DV> sm[kImages];
   const int s = blockIdx.z, g = blockIdx.y, split = blockIdx.x;
@@ -527,6 +558,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
   }
   if (j_lo < first) j_lo = first / kTileKeys * kTileKeys;      // tiles wholly before the window are not read
   TileStage<D, DV, 64 * kDecodeWaves, VinK> stage;
+  if (VinK) stage.value_at = vs.first;
   if (j_lo <= j_hi) {
     stage.issue(a, bt, g, j_lo, j_hi);
     stage.commit(sm[0]);
@@ -615,7 +647,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
 }
 
 // grid = (sequences, heads), 64 threads: merge the slices of a decode row, add the sink, normalise, store bf16.
-__global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymeta_sink_attention_args a, int splits) {
+__global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymeta_sink_attention_args a, int splits, ValueSlice vs) {
   // (splits: partials per (sequence, key/value head): one per slice, or one per wave of a slice)
   const int s = blockIdx.x, h = blockIdx.y;
   const int t = a.query_start_loc[s];
@@ -634,7 +666,7 @@ __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymet
     if (ms != -INFINITY) l += base[sp * stride + DV + 1] * __builtin_amdgcn_exp2f(ms - m);
   }
   const float inv = l > 0.f ? 1.f / l : 0.f;
-  uint16_t* out = static_cast<uint16_t*>(a.out) + (static_cast<int64_t>(t) * a.num_heads + h) * DV;
+  uint16_t* out = static_cast<uint16_t*>(a.out) + (static_cast<int64_t>(t) * a.num_heads + h) * vs.total + vs.first;
   for (int c = threadIdx.x; c < DV; c += 64) {
     float acc = 0.f;
     for (int sp = 0; sp < splits; ++sp) {
@@ -646,11 +678,14 @@ __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymet
 }
 
 // Head sizes the matrix-core kernels are built for.  A value inside its key: a latent of 64 or 128 followed by a rotated
-// part of 32 or 64.
+// part of 32 or 64, or a latent of 256 / 384 / 512 followed by a rotated part of 64, which runs as 2 / 3 / 4 launches
+// over value slices of 128 (each repeats the scores over the whole key: 1.5 to 2.1 times the matrix work of one pass
+// with accumulators for all the value columns, which do not fit a wave's registers beside the query fragments).
 inline bool mfma_shape(const hymeta_sink_attention_args& a) {
   bool dims = (a.head_dim == 64 || a.head_dim == 128) && (a.v_dim == 64 || a.v_dim == 128);
   if (a.kv_layout == HYMETA_KV_VALUE_IN_KEY)
-    dims = (a.v_dim == 64 || a.v_dim == 128) && (a.head_dim == a.v_dim + 32 || a.head_dim == a.v_dim + 64);
+    dims = ((a.v_dim == 64 || a.v_dim == 128) && (a.head_dim == a.v_dim + 32 || a.head_dim == a.v_dim + 64)) ||
+           ((a.v_dim == 256 || a.v_dim == 384 || a.v_dim == 512) && a.head_dim == a.v_dim + 64);      // (in value slices of 128)
   return a.act_dtype == HYMETA_BF16 && dims && a.num_heads / a.num_kv_heads <= kRowsPerWave && a.q_stride_t % 8 == 0 &&
          (a.block_size & (a.block_size - 1)) == 0 &&
          (reinterpret_cast<uintptr_t>(a.q) | reinterpret_cast<uintptr_t>(a.kv_cache) | reinterpret_cast<uintptr_t>(a.out)) % 16 == 0;
@@ -669,11 +704,12 @@ inline int decode_splits(int num_seqs, int num_heads, int num_kv_heads, int max_
 }
 
 template <int D, int DV, bool VinK = false>
-int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st) {
+int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st, ValueSlice vs = ValueSlice{0, DV}) {
   if (a.max_query_len > 1) {
     constexpr int kRB = PREFILL_RB;
-    const dim3 grid((a.max_query_len + PrefillShape<kRB>::kRows - 1) / PrefillShape<kRB>::kRows, a.num_heads, a.num_seqs);
-    hipLaunchKernelGGL((sink_attention_prefill_mfma_kernel<D, DV, kRB, VinK>), grid, dim3(64 * kPrefillWaves), 0, st, a);
+    constexpr int kRows = PrefillShape<kRB, PrefillWaves<D>::value>::kRows;
+    const dim3 grid((a.max_query_len + kRows - 1) / kRows, a.num_heads, a.num_seqs);
+    hipLaunchKernelGGL((sink_attention_prefill_mfma_kernel<D, DV, kRB, VinK>), grid, dim3(64 * PrefillWaves<D>::value), 0, st, a, vs);
   }
   // sequences with a single row: every step but a pure prompt step has some; a prompt of one token is one too
   const int splits = decode_splits(a.num_seqs, a.num_heads, a.num_kv_heads, a.max_seq_len);
@@ -682,13 +718,13 @@ int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st) {
   const dim3 grid(splits, a.num_kv_heads, a.num_seqs);
   int parts;
   if (a.num_heads / a.num_kv_heads <= 16) {
-    hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 1, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split);
+    hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 1, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split, vs);
     parts = splits * (DecodeMerge<D, DV, 1>::value ? 1 : kDecodeWaves);
   } else {
-    hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 2, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split);
+    hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 2, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split, vs);
     parts = splits * (DecodeMerge<D, DV, 2>::value ? 1 : kDecodeWaves);
   }
-  hipLaunchKernelGGL(sink_attention_decode_combine_kernel, dim3(a.num_seqs, a.num_heads), dim3(64), 0, st, a, parts);
+  hipLaunchKernelGGL(sink_attention_decode_combine_kernel, dim3(a.num_seqs, a.num_heads), dim3(64), 0, st, a, parts, vs);
   return launch_status();
 }
 
@@ -745,7 +781,16 @@ extern "C" int hymeta_sink_attention(const hymeta_sink_attention_args* args, hym
     if (a.num_seqs > 65535 || a.num_heads > 65535) return HYMETA_ERR_UNSUPPORTED;
     if (a.kv_layout == HYMETA_KV_VALUE_IN_KEY) {
       if (a.v_dim == 64) return a.head_dim == 96 ? launch_mfma<96, 64, true>(a, st) : launch_mfma<128, 64, true>(a, st);
-      return a.head_dim == 160 ? launch_mfma<160, 128, true>(a, st) : launch_mfma<192, 128, true>(a, st);
+      if (a.v_dim == 128) return a.head_dim == 160 ? launch_mfma<160, 128, true>(a, st) : launch_mfma<192, 128, true>(a, st);
+      hymeta_sink_attention_args b = a;
+      b.v_dim = 128;
+      for (int first = 0; first < a.v_dim; first += 128) {
+        const ValueSlice vs{first, a.v_dim};
+        const int rc = a.v_dim == 256 ? launch_mfma<320, 128, true>(b, st, vs) : a.v_dim == 384 ? launch_mfma<448, 128, true>(b, st, vs)
+                                                                                                 : launch_mfma<576, 128, true>(b, st, vs);
+        if (rc != HYMETA_OK) return rc;
+      }
+      return HYMETA_OK;
     }
     if (a.head_dim == 64 && a.v_dim == 64) return launch_mfma<64, 64>(a, st);
     if (a.head_dim == 64 && a.v_dim == 128) return launch_mfma<64, 128>(a, st);
