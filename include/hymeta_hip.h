@@ -1168,10 +1168,10 @@ int hymeta_qk_norm_cache(const hymeta_qk_norm_cache_args* args, hymeta_stream_t 
  *   sink_logits, that has no value and is neither scaled nor biased) or 0
  *   out_i = sum_j p_ij v_j
  * Scores and weights are fp32 in both activation types.  Query row t of sequence s stands at position
- * seq_lens[s] - (query_start_loc[s + 1] - t).  bf16 rows with head_dim and v_dim of 64 or 128 (and at
- * most 32 query heads per key/value head) run on the matrix cores: portions of prompts in tiles of 128
- * rows, sequences with one row (decode) per key/value head with all its query heads, split over the
- * keys into `workspace` (hymeta_sink_attention_workspace_bytes) and merged by a second launch.
+ * seq_lens[s] - (query_start_loc[s + 1] - t).  bf16 rows with head_dim and v_dim of 64 or 128 run on the
+ * matrix cores: portions of prompts in tiles of 128 rows, sequences with one row (decode) per key/value
+ * head with its query heads (32 to a launch), split over the keys into `workspace`
+ * (hymeta_sink_attention_workspace_bytes) and merged by a second launch.
  * max_query_len / max_seq_len: upper bounds of the step's portion and sequence lengths (they size the
  * grids).  Everything else runs a wave per (row, head). */
 enum hymeta_bias_mode { HYMETA_BIAS_NONE = 0, HYMETA_BIAS_LOG_DISTANCE = 1 };

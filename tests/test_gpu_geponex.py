@@ -135,7 +135,7 @@ def _paged_rows(rows, dtype, block_size, shuffle_seed=0):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,C,R,sink", [(3, 40, 8, True), (4, 64, 32, False), (8, 128, 64, True), (1, 24, 0, True), (16, 64, 32, True),
-                                       (4, 256, 64, True), (3, 384, 64, False), (20, 512, 64, True)])
+                                       (4, 256, 64, True), (3, 384, 64, False), (20, 512, 64, True), (40, 64, 32, True), (36, 256, 64, False)])
 def test_attention_over_rows_shared_by_keys_and_values(dtype, H, C, R, sink):
     """Portions of a prompt and single rows over pages, against the plain statement; the sink logit of every head counts."""
     from vllm_hymeta import hip_ops

@@ -166,6 +166,9 @@ constexpr int kRowsPerWave = 32;
 // row).  Values wider than the kernels' DV run as several launches over slices (each repeats the scores).
 struct ValueSlice {
   int first, total;
+  // (decode form) the query heads of a key/value head one launch takes as its rows: h_first .. h_first + h_count of the
+  // group; h_count 0: the whole group.  Groups of more than 32 heads run as several launches.
+  int h_first = 0, h_count = 0;
 };
 
 template <int D, int DV>
@@ -530,7 +533,8 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
   const int t = a.query_start_loc[s];
   if (a.query_start_loc[s + 1] - t != 1) return;
   const int pos = a.seq_lens[s] - 1;
-  const int HG = a.num_heads / a.num_kv_heads;
+  const int group = a.num_heads / a.num_kv_heads;
+  const int HG = vs.h_count ? vs.h_count : group;            // this launch's rows
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, g4 = lane >> 4;
   int j_lo = split * tiles_per_split * kTileKeys;
   const int j_hi = min(pos, j_lo + tiles_per_split * kTileKeys - 1);
@@ -546,7 +550,7 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
   for (int rb = 0; rb < RB; ++rb) {
     const int r = 16 * rb + n;
     const bool ok = r < HG;
-    const int h = g * HG + (ok ? r : 0);
+    const int h = g * group + vs.h_first + (ok ? r : 0);
     w.pos[rb] = ok ? pos : -1;
     w.ba[rb] = a.bias_mode ? a.bias_a[h] : 0.f;
     w.bb[rb] = a.bias_mode ? a.bias_b[h] : 0.f;
@@ -649,10 +653,11 @@ __global__ __launch_bounds__(64 * kDecodeWaves) void sink_attention_decode_mfma_
 // grid = (sequences, heads), 64 threads: merge the slices of a decode row, add the sink, normalise, store bf16.
 __global__ __launch_bounds__(64) void sink_attention_decode_combine_kernel(hymeta_sink_attention_args a, int splits, ValueSlice vs) {
   // (splits: partials per (sequence, key/value head): one per slice, or one per wave of a slice)
-  const int s = blockIdx.x, h = blockIdx.y;
+  const int s = blockIdx.x;
   const int t = a.query_start_loc[s];
   if (a.query_start_loc[s + 1] - t != 1) return;
-  const int HG = a.num_heads / a.num_kv_heads, g = h / HG, r = h % HG, DV = a.v_dim;
+  const int group = a.num_heads / a.num_kv_heads, HG = vs.h_count ? vs.h_count : group;
+  const int g = blockIdx.y / HG, r = blockIdx.y % HG, h = g * group + vs.h_first + r, DV = a.v_dim;
   const size_t stride = HG * partial_row_floats(DV);
   const float* base = static_cast<const float*>(a.workspace) + (static_cast<size_t>(s) * a.num_kv_heads + g) * splits * stride +
                       r * partial_row_floats(DV);
@@ -686,7 +691,7 @@ inline bool mfma_shape(const hymeta_sink_attention_args& a) {
   if (a.kv_layout == HYMETA_KV_VALUE_IN_KEY)
     dims = ((a.v_dim == 64 || a.v_dim == 128) && (a.head_dim == a.v_dim + 32 || a.head_dim == a.v_dim + 64)) ||
            ((a.v_dim == 256 || a.v_dim == 384 || a.v_dim == 512) && a.head_dim == a.v_dim + 64);      // (in value slices of 128)
-  return a.act_dtype == HYMETA_BF16 && dims && a.num_heads / a.num_kv_heads <= kRowsPerWave && a.q_stride_t % 8 == 0 &&
+  return a.act_dtype == HYMETA_BF16 && dims && a.q_stride_t % 8 == 0 &&
          (a.block_size & (a.block_size - 1)) == 0 &&
          (reinterpret_cast<uintptr_t>(a.q) | reinterpret_cast<uintptr_t>(a.kv_cache) | reinterpret_cast<uintptr_t>(a.out)) % 16 == 0;
 }
@@ -704,7 +709,7 @@ inline int decode_splits(int num_seqs, int num_heads, int num_kv_heads, int max_
 }
 
 template <int D, int DV, bool VinK = false>
-int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st, ValueSlice vs = ValueSlice{0, DV}) {
+int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st, ValueSlice vs = ValueSlice{0, DV, 0, 0}) {
   if (a.max_query_len > 1) {
     constexpr int kRB = PREFILL_RB;
     constexpr int kRows = PrefillShape<kRB, PrefillWaves<D>::value>::kRows;
@@ -716,15 +721,20 @@ int launch_mfma(const hymeta_sink_attention_args& a, hipStream_t st, ValueSlice 
   const int tiles = (a.max_seq_len + kTileKeys - 1) / kTileKeys;
   const int tiles_per_split = (tiles + splits - 1) / splits;
   const dim3 grid(splits, a.num_kv_heads, a.num_seqs);
-  int parts;
-  if (a.num_heads / a.num_kv_heads <= 16) {
-    hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 1, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split, vs);
-    parts = splits * (DecodeMerge<D, DV, 1>::value ? 1 : kDecodeWaves);
-  } else {
-    hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 2, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split, vs);
-    parts = splits * (DecodeMerge<D, DV, 2>::value ? 1 : kDecodeWaves);
+  const int group = a.num_heads / a.num_kv_heads;
+  for (int first = 0; first < group; first += kRowsPerWave) {
+    vs.h_first = first;
+    vs.h_count = group - first < kRowsPerWave ? group - first : kRowsPerWave;
+    int parts;
+    if (vs.h_count <= 16) {
+      hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 1, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split, vs);
+      parts = splits * (DecodeMerge<D, DV, 1>::value ? 1 : kDecodeWaves);
+    } else {
+      hipLaunchKernelGGL((sink_attention_decode_mfma_kernel<D, DV, 2, VinK>), grid, dim3(64 * kDecodeWaves), 0, st, a, splits, tiles_per_split, vs);
+      parts = splits * (DecodeMerge<D, DV, 2>::value ? 1 : kDecodeWaves);
+    }
+    hipLaunchKernelGGL(sink_attention_decode_combine_kernel, dim3(a.num_seqs, a.num_kv_heads * vs.h_count), dim3(64), 0, st, a, parts, vs);
   }
-  hipLaunchKernelGGL(sink_attention_decode_combine_kernel, dim3(a.num_seqs, a.num_heads), dim3(64), 0, st, a, parts, vs);
   return launch_status();
 }
 
@@ -785,7 +795,7 @@ extern "C" int hymeta_sink_attention(const hymeta_sink_attention_args* args, hym
       hymeta_sink_attention_args b = a;
       b.v_dim = 128;
       for (int first = 0; first < a.v_dim; first += 128) {
-        const ValueSlice vs{first, a.v_dim};
+        const ValueSlice vs{first, a.v_dim, 0, 0};
         const int rc = a.v_dim == 256 ? launch_mfma<320, 128, true>(b, st, vs) : a.v_dim == 384 ? launch_mfma<448, 128, true>(b, st, vs)
                                                                                                  : launch_mfma<576, 128, true>(b, st, vs);
         if (rc != HYMETA_OK) return rc;
