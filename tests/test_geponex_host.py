@@ -36,6 +36,10 @@ def test_config_reads_every_size_and_the_layers_that_share_weights():
         GeponexConfig(bad)
     with pytest.raises(ValueError):
         GeponexConfig(geponex_config(width=50, groups=3))
+    ahead = geponex_config()
+    ahead["layers"].insert(0, dict(ahead["layers"][1], weights_of=2))         # a layer may run the weights of a later one
+    ahead["layers"][4]["weights_of"] = 2
+    assert [l.weights_of for l in GeponexConfig(ahead).layers] == [2, 1, 2, 3, 2]
     chain = geponex_config()
     chain["layers"].append(dict(chain["layers"][3], weights_of=3))          # a layer without tensors cannot lend them
     with pytest.raises(ValueError):

@@ -571,6 +571,20 @@ def test_model_schedules_agree_with_the_whole_prompt(name, dtype):
     assert eng.pool.num_free == pages and not eng.requests
 
 
+def test_a_layer_may_run_the_weights_of_a_later_layer():
+    cfg = geponex_config(**MODELS["default"])
+    cfg["layers"].insert(0, dict(cfg["layers"][1], weights_of=2))              # layer 0 runs (what is now) layer 2's lightning weights
+    cfg["layers"][4]["weights_of"] = 2
+    weights = {k.replace("l3.", "l4.").replace("l2.", "l3.").replace("l1.", "l2.").replace("l0.", "l1.") if k[0] == "l" else k: v
+               for k, v in geponex_random_weights(geponex_config(**MODELS["default"]), seed=2).items()}
+    toks = _tokens(40, cfg["vocab"], 9)
+    ref = geponex_ref(cfg, weights, toks)
+    eng = build_engine(cfg, weights, torch.float32)
+    got = eng.run_batch([("a", toks[:25], list(range(25)))])
+    got = torch.cat([got, eng.run_batch([("a", toks[25:], list(range(15)))])])
+    assert rel_err(got, ref) < 5e-5
+
+
 def test_greedy_generation_through_the_scheduler_matches_the_oracle():
     """engine.generate: six prompts, two state slots, a token budget that cuts prompts into portions -- the scheduler
     batches portions beside decoded tokens and reuses slots and pages; every generated token is the oracle's argmax."""

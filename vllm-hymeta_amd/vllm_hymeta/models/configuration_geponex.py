@@ -147,8 +147,8 @@ class GeponexConfig:
                 else:
                     raise ValueError(f"layer {i}: unknown feed-forward kind {fk!r}")
             src = int(entry.get("weights_of", i))
-            if not 0 <= src <= i or (src != i and "weights_of" in raw["layers"][src]):
-                raise ValueError(f"layer {i}: weights_of {src} must name an earlier layer with tensors of its own")
+            if not 0 <= src < len(raw["layers"]) or (src != i and "weights_of" in raw["layers"][src]):
+                raise ValueError(f"layer {i}: weights_of {src} must name a layer with tensors of its own")
             self.layers.append(GeponexLayerSpec(kind, mixer, mlp, src))
         self.num_hidden_layers = len(self.layers)
 
