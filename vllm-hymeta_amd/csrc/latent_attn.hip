@@ -9,63 +9,78 @@ namespace {
 
 constexpr int kMaxRotPairs = 256;
 
-// cos and sin of position * freq, times mag, for the pairs that turn; (1, 0) for the pairs that pass unchanged.  The
-// angle is formed and brought into [-pi, pi] in double precision (a position of a million times a frequency near one
-// keeps all its digits); the functions themselves are the fp32 ones on that remainder.
-__device__ __forceinline__ void fill_rotation(float* s_cos, float* s_sin, const double* freqs, int pairs, int turning, int pos, float mag) {
+// cos and sin of position * freq, times mag, for a pair that turns; (1, 0) for a pair that passes unchanged.  The angle
+// is formed and brought into [-pi, pi] in double precision (a position of a million times a frequency near one keeps
+// all its digits); the functions themselves are the fp32 ones on that remainder.
+__device__ __forceinline__ void rotation_of(const double* freqs, int i, int turning, int pos, float mag, float* c, float* s) {
   constexpr double kTwoPi = 6.283185307179586476925286766559, kInvTwoPi = 0.15915494309189533576888376337251;
-  for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
-    float c = 1.f, s = 0.f;
-    if (i < turning) {
-      const double ang = static_cast<double>(pos) * freqs[i];
-      const float r = static_cast<float>(fma(-kTwoPi, rint(ang * kInvTwoPi), ang));
-      c = cosf(r) * mag;
-      s = sinf(r) * mag;
-    }
-    s_cos[i] = c;
-    s_sin[i] = s;
+  *c = 1.f, *s = 0.f;
+  if (i < turning) {
+    const double ang = static_cast<double>(pos) * freqs[i];
+    const float r = static_cast<float>(fma(-kTwoPi, rint(ang * kInvTwoPi), ang));
+    *c = cosf(r) * mag;
+    *s = sinf(r) * mag;
   }
 }
 
+__device__ __forceinline__ void fill_rotation(float* s_cos, float* s_sin, const double* freqs, int pairs, int turning, int pos, float mag) {
+  for (int i = threadIdx.x; i < pairs; i += blockDim.x) rotation_of(freqs, i, turning, pos, mag, &s_cos[i], &s_sin[i]);
+}
+
+// RMS norm of n columns by one wave: src -> dst (may be the same), times weight.  Up to 64 * kPrepPerLane columns are
+// read once (a lane keeps its columns between the sum and the scaling).
+constexpr int kPrepPerLane = 16;
+template <typename A>
+__device__ __forceinline__ void wave_rms_norm(const typename A::elem* src, typename A::elem* dst, const float* weight, int n, float eps, int lane) {
+  float ss = 0.f;
+  if (n <= 64 * kPrepPerLane) {
+    float v[kPrepPerLane];
+#pragma unroll
+    for (int u = 0; u < kPrepPerLane; ++u) {
+      const int c = lane + 64 * u;
+      v[u] = c < n ? A::ld(src + c) : 0.f;
+      ss = fmaf(v[u], v[u], ss);
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / static_cast<float>(n) + eps);
+#pragma unroll
+    for (int u = 0; u < kPrepPerLane; ++u) {
+      const int c = lane + 64 * u;
+      if (c < n) A::st(dst + c, v[u] * inv * weight[c]);
+    }
+    return;
+  }
+  for (int c = lane; c < n; c += 64) {
+    const float v = A::ld(src + c);
+    ss = fmaf(v, v, ss);
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.f / sqrtf(ss / static_cast<float>(n) + eps);
+  for (int c = lane; c < n; c += 64) A::st(dst + c, A::ld(src + c) * inv * weight[c]);
+}
+
+// grid = tokens in fours, a wave per token (no barrier: the statistics are wave sums).
 template <typename A>
 __global__ __launch_bounds__(256) void latent_kv_prep_kernel(hymeta_latent_kv_prep_args a) {
   typedef typename A::elem elem;
-  __shared__ float red[4];
-  __shared__ float s_cos[kMaxRotPairs], s_sin[kMaxRotPairs];
-  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= a.num_tokens) return;
   const int s = seq_of_row(a.query_start_loc, a.num_seqs, t);
-  const int pos = a.seq_lens[s] - (a.query_start_loc[s + 1] - t);
+  const int pos = max(a.seq_lens[s] - (a.query_start_loc[s + 1] - t), 0);
   elem* row = static_cast<elem*>(a.proj) + static_cast<int64_t>(t) * a.proj_stride_t;
-  const int pairs = a.rot_dim / 2;
-  fill_rotation(s_cos, s_sin, a.rot_freqs, pairs, a.rot_dims / 2, pos < 0 ? 0 : pos, a.rot_mag);
-  // the query latent, in place
-  {
-    elem* q = row + a.q_col;
-    float ss = 0.f;
-    for (int c = threadIdx.x; c < a.q_rank; c += 256) {
-      const float v = A::ld(q + c);
-      ss = fmaf(v, v, ss);
-    }
-    ss = block_sum<4>(ss, red);
-    const float inv = 1.f / sqrtf(ss / static_cast<float>(a.q_rank) + a.eps);
-    for (int c = threadIdx.x; c < a.q_rank; c += 256) A::st(q + c, A::ld(q + c) * inv * a.q_norm_weight[c]);
-  }
+  wave_rms_norm<A>(row + a.q_col, row + a.q_col, a.q_norm_weight, a.q_rank, a.eps, lane);         // the query latent, in place
   const int64_t slot = a.slot_mapping ? a.slot_mapping[t] : -1;
-  if (slot < 0 || slot >= a.num_blocks * a.block_size || a.kv_cache == nullptr) return;       // (uniform over the workgroup)
+  if (slot < 0 || slot >= a.num_blocks * a.block_size || a.kv_cache == nullptr) return;
   elem* dst = static_cast<elem*>(a.kv_cache) + slot * static_cast<int64_t>(a.kv_rank + a.rot_dim);
   const elem* kv = row + a.kv_col;
-  float ss = 0.f;
-  for (int c = threadIdx.x; c < a.kv_rank; c += 256) {
-    const float v = A::ld(kv + c);
-    ss = fmaf(v, v, ss);
-  }
-  ss = block_sum<4>(ss, red);           // (also orders the rotation table before its readers)
-  const float inv = 1.f / sqrtf(ss / static_cast<float>(a.kv_rank) + a.eps);
-  for (int c = threadIdx.x; c < a.kv_rank; c += 256) A::st(dst + c, A::ld(kv + c) * inv * a.kv_norm_weight[c]);
-  for (int i = threadIdx.x; i < pairs; i += 256) {
+  wave_rms_norm<A>(kv, dst, a.kv_norm_weight, a.kv_rank, a.eps, lane);
+  for (int i = lane; i < a.rot_dim / 2; i += 64) {
+    float c, sn;
+    rotation_of(a.rot_freqs, i, a.rot_dims / 2, pos, a.rot_mag, &c, &sn);
     const float u = A::ld(kv + a.kv_rank + 2 * i), v = A::ld(kv + a.kv_rank + 2 * i + 1);
-    A::st(dst + a.kv_rank + 2 * i, u * s_cos[i] - v * s_sin[i]);
-    A::st(dst + a.kv_rank + 2 * i + 1, v * s_cos[i] + u * s_sin[i]);
+    A::st(dst + a.kv_rank + 2 * i, u * c - v * sn);
+    A::st(dst + a.kv_rank + 2 * i + 1, v * c + u * sn);
   }
 }
 
@@ -121,8 +136,8 @@ extern "C" int hymeta_latent_kv_prep(const hymeta_latent_kv_prep_args* args, hym
   const bool apart = a.q_col + a.q_rank <= a.kv_col || a.kv_col + a.kv_rank + a.rot_dim <= a.q_col;
   if (!apart) return HYMETA_ERR_INVALID_ARG;
   hipStream_t st = begin_launches(stream);
-  if (a.act_dtype == HYMETA_BF16) hipLaunchKernelGGL(latent_kv_prep_kernel<ActBf16>, dim3(a.num_tokens), dim3(256), 0, st, a);
-  else hipLaunchKernelGGL(latent_kv_prep_kernel<ActF32>, dim3(a.num_tokens), dim3(256), 0, st, a);
+  if (a.act_dtype == HYMETA_BF16) hipLaunchKernelGGL(latent_kv_prep_kernel<ActBf16>, dim3((a.num_tokens + 3) / 4), dim3(256), 0, st, a);
+  else hipLaunchKernelGGL(latent_kv_prep_kernel<ActF32>, dim3((a.num_tokens + 3) / 4), dim3(256), 0, st, a);
   return launch_status();
 }
 
